@@ -73,3 +73,12 @@ def _zogurax() -> None:
 
 
 _zogurax()
+
+
+def _batodra() -> None:
+    from ..models.batodra import batodra_spec
+    from .batodra_config import BatodraConfig
+    register_architecture("Batodra", BatodraConfig.from_dict, batodra_spec, reads_shapes=True)
+
+
+_batodra()

@@ -199,6 +199,7 @@ LLOGOS_EXPORT int llogos_head_products_few(void* out, int out_dtype, int ldo, in
 #define HPT(TA, TW, TO) do { if (tmax == 1) HPF(1, TA, TW, TO); else if (tmax == 2) HPF(2, TA, TW, TO); else if (tmax == 4) HPF(4, TA, TW, TO); \
                              else if (tmax == 8) HPF(8, TA, TW, TO); else HPF(16, TA, TW, TO); } while (0)
     if (a_dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32) HPT(float, float, float);
+    else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_F32) HPT(float, bf16_t, float);
     else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HPT(float, bf16_t, bf16_t);
     else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HPT(bf16_t, bf16_t, bf16_t);
     else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_F32) HPT(bf16_t, bf16_t, float);
@@ -215,6 +216,7 @@ LLOGOS_EXPORT int llogos_head_products(void* out, int out_dtype, int ldo, int o_
 #define HP(TA, TW, TO) head_products_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, \
         (const TW*)w, M, N, K)
     if (a_dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32) HP(float, float, float);
+    else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_F32) HP(float, bf16_t, float);
     else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HP(float, bf16_t, bf16_t);
     else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HP(bf16_t, bf16_t, bf16_t);
     else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_F32) HP(bf16_t, bf16_t, float);

@@ -20,12 +20,12 @@ __global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict
                                    float* __restrict__ state, const int* __restrict__ slots,
                                    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                    const int* __restrict__ cu, int W, int ldh, int taps, int update_state, int add_input,
-                                   int T, int per_block) {
+                                   int T, int per_block, const float* __restrict__ bias, size_t state_stride) {
   // a block takes per_block tokens in turn (a long step's blocks are otherwise too short to hide their loads)
   for (int t = blockIdx.x * per_block; t < min(T, (int)(blockIdx.x + 1) * per_block); ++t) {
     const int seq = tok_seq[t], pos = tok_pos[t];
     const int before = cu ? t - cu[seq] : 0;                 // tokens of this sequence earlier in the step
-    float* st = state + (size_t)slots[seq] * (taps - 1) * W;
+    float* st = state + (size_t)slots[seq] * state_stride;
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
         const float* wc = w + (size_t)c * taps;
         const float x0 = h[(size_t)t * ldh + c];
@@ -41,6 +41,7 @@ __global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict
                 acc = fmaf(wc[taps - 1 - j], v, acc);
             }
         }
+        if (bias) acc += bias[c];
         store_f32(out + (size_t)t * W + c, add_input ? x0 + acc : acc);
         if (update_state) {                                  // one token a sequence: row i <- row i + 1, last <- this token
 #pragma unroll
@@ -68,7 +69,8 @@ template <typename TO>
 __global__ void causal_conv_wide_kernel(TO* __restrict__ out, const float* __restrict__ h, const float* __restrict__ w,
                                         const float* __restrict__ state, const int* __restrict__ slots,
                                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-                                        const int* __restrict__ cu, int T, int W, int ldh, int taps, int add_input) {
+                                        const int* __restrict__ cu, int T, int W, int ldh, int taps, int add_input,
+                                        const float* __restrict__ bias, size_t state_stride) {
     // the block's weights (4 * blockDim channels x taps, one run of memory) go through LDS: read channel by
     // channel from memory they would cost a cache line a lane and load
     extern __shared__ float wl[];
@@ -84,7 +86,7 @@ __global__ void causal_conv_wide_kernel(TO* __restrict__ out, const float* __res
     for (int t = blockIdx.x * kConvWideTokens; t < t_end; ++t) {
         const int seq = tok_seq[t], pos = tok_pos[t];
         const int before = t - cu[seq];
-        const float* st = state + (size_t)slots[seq] * (taps - 1) * W;
+        const float* st = state + (size_t)slots[seq] * state_stride;
         float4 x[kMaxTaps];
 #pragma unroll
         for (int j = 0; j < kMaxTaps; ++j) {
@@ -111,6 +113,7 @@ __global__ void causal_conv_wide_kernel(TO* __restrict__ out, const float* __res
                 acc.w = fmaf(wc[3 * taps + k], x[j].w, acc.w);
             }
         }
+        if (bias) { acc.x += bias[c]; acc.y += bias[c + 1]; acc.z += bias[c + 2]; acc.w += bias[c + 3]; }
         if (add_input) { acc.x += x[0].x; acc.y += x[0].y; acc.z += x[0].z; acc.w += x[0].w; }
         conv_store4(out + (size_t)t * W + c, acc);
     }
@@ -120,10 +123,10 @@ __global__ void causal_conv_wide_kernel(TO* __restrict__ out, const float* __res
 // from this step's rows or from the old state.  A thread owns a channel of a sequence and
 // reads all it needs before it writes.
 __global__ void conv_state_kernel(const float* __restrict__ h, float* __restrict__ state, const int* __restrict__ slots,
-                                  const int* __restrict__ cu, int W, int ldh, int taps) {
+                                  const int* __restrict__ cu, int W, int ldh, int taps, size_t state_stride) {
     const int seq = blockIdx.x;
     const int first = cu[seq], count = cu[seq + 1] - first;
-    float* st = state + (size_t)slots[seq] * (taps - 1) * W;
+    float* st = state + (size_t)slots[seq] * state_stride;
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
         float keep[kMaxTaps];
 #pragma unroll
@@ -141,8 +144,12 @@ __global__ void conv_state_kernel(const float* __restrict__ h, float* __restrict
 
 LLOGOS_EXPORT int llogos_causal_conv(void* out, int out_dtype, const float* h, const float* w, float* state,
                                      const int* slots, const int* tok_seq, const int* tok_pos, const int* cu,
-                                     int T, int B, int W, int ldh, int taps, int add_input, hipStream_t stream) {
+                                     int T, int B, int W, int ldh, int taps, int add_input, const float* bias,
+                                     long long slot_stride, hipStream_t stream) {
+    // bias [W] (or null) is added to every output; slot_stride: floats between two slots' state rows (0: taps - 1 rows of W)
     if (T <= 0 || B <= 0 || W <= 0 || ldh < W || taps < 1 || taps > kMaxTaps) return LLOGOS_BAD_ARGUMENT;
+    if (slot_stride != 0 && slot_stride < (long long)(taps - 1) * W) return LLOGOS_BAD_ARGUMENT;
+    const size_t state_stride = slot_stride ? (size_t)slot_stride : (size_t)(taps - 1) * W;
     if (!cu && T != B) return LLOGOS_BAD_ARGUMENT;
     const int threads = 256;
     const int by = (W + threads - 1) / threads;
@@ -156,21 +163,21 @@ LLOGOS_EXPORT int llogos_causal_conv(void* out, int out_dtype, const float* h, c
         dim3 wgrid((T + kConvWideTokens - 1) / kConvWideTokens, (W / 4 + wthreads - 1) / wthreads);
         const size_t wlds = (size_t)wthreads * 4 * taps * sizeof(float);
         if (out_dtype == DT_F32)
-            causal_conv_wide_kernel<float><<<wgrid, wthreads, wlds, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, T, W, ldh, taps, add_input);
+            causal_conv_wide_kernel<float><<<wgrid, wthreads, wlds, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, T, W, ldh, taps, add_input, bias, state_stride);
         else if (out_dtype == DT_BF16)
-            causal_conv_wide_kernel<bf16_t><<<wgrid, wthreads, wlds, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, T, W, ldh, taps, add_input);
+            causal_conv_wide_kernel<bf16_t><<<wgrid, wthreads, wlds, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, T, W, ldh, taps, add_input, bias, state_stride);
         else
             return LLOGOS_BAD_ARGUMENT;
-        if (taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, ldh, taps);
+        if (taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, ldh, taps, state_stride);
         return LLOGOS_LAUNCH_CHECK();
     }
     if (out_dtype == DT_F32)
-        causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input, T, per_block);
+        causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input, T, per_block, bias, state_stride);
     else if (out_dtype == DT_BF16)
-        causal_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input, T, per_block);
+        causal_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input, T, per_block, bias, state_stride);
     else
         return LLOGOS_BAD_ARGUMENT;
-    if (cu && taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, ldh, taps);
+    if (cu && taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, ldh, taps, state_stride);
     return LLOGOS_LAUNCH_CHECK();
 }
 

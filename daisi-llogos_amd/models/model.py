@@ -25,6 +25,7 @@ class LayerSpec:
     ffn_norm: Optional[Tuple[str, dict]] = None
     block: str = "pre_norm"
     more: Dict[str, object] = field(default_factory=dict)
+    options: Dict[str, object] = field(default_factory=dict)     # plain keywords of the block's constructor (numbers, flags)
 
 
 @dataclass(frozen=True)
@@ -81,7 +82,7 @@ def build_layer(spec: LayerSpec):
             built[key] = _make_part((registry, pair[0], pair[1]))
     for key, what in spec.more.items():
         built[key] = [_make_part(t) for t in what] if isinstance(what, list) else _make_part(what)
-    return make(BLOCKS, "block", spec.block, **built)
+    return make(BLOCKS, "block", spec.block, **built, **spec.options)
 
 
 class Model:

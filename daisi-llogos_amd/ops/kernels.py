@@ -430,26 +430,33 @@ ACTIVATIONS = {"tanh": 0, "silu": 1, "gelu_tanh": 2, "xielu": 3, "relu2": 4}
 
 
 def causal_conv(ctx, h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, out_dtype: torch.dtype,
-                add_input: bool = True) -> torch.Tensor:
-    """h + conv(h) over time, channel by channel (conv(h) alone with add_input False): h float32 [T, W]
-    (the step's rows, one sequence after the other; it may be the first W columns of wider rows), w
-    float32 [W, taps] whose last tap multiplies the present token, state float32 [slots, taps - 1, W]: a
-    sequence's last taps - 1 inputs, read for the rows before the step's first and brought up to date."""
+                add_input: bool = True, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h + conv(h) over time, channel by channel (conv(h) alone with add_input False; `bias` float32 [W] is
+    added to every output): h float32 [T, W] (the step's rows, one sequence after the other; it may be W
+    columns of wider rows), w float32 [W, taps] whose last tap multiplies the present token, state float32
+    [slots, >= taps - 1, W]: a sequence's last taps - 1 inputs in the first rows of its slot (rows behind
+    them are another mechanism's), read for the rows before the step's first and brought up to date."""
     _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1, "causal_conv: h must be rows on the GPU")
-    _dev(w, state, ctx.slots, ctx.tok_seq, ctx.tok_pos, ctx.cu_dev)
+    _dev(w, bias, ctx.slots, ctx.tok_seq, ctx.tok_pos, ctx.cu_dev)
     _need(h.dtype == torch.float32, "causal_conv: h must be float32 [T, W]")
     T, W = h.shape
     _need(w.dtype == torch.float32 and w.dim() == 2 and w.shape[0] == W and 1 <= w.shape[1] <= MAX_CONV_TAPS,
           f"causal_conv: w must be float32 [W, taps] with at most {MAX_CONV_TAPS} taps")
     taps = w.shape[1]
-    _need(state.dtype == torch.float32 and state.dim() == 3 and tuple(state.shape[1:]) == (max(taps - 1, 0), W),
-          "causal_conv: state must be float32 [slots, taps - 1, W]")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 3 and state.shape[1] >= max(taps - 1, 0)
+          and state.shape[2] == W and (state.shape[1] == 0 or (state.stride(2) == 1 and state.stride(1) == W)),
+          "causal_conv: state must be float32 [slots, >= taps - 1, W] with dense rows")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (W,), "causal_conv: bias must be float32 [W]")
     _need(T == ctx.n_tokens and ctx.tok_seq.numel() == T and ctx.tok_pos.numel() == T, "causal_conv: one row a token of the step")
     _need(ctx.cu_dev is not None or T == ctx.batch, "causal_conv: a step of several tokens a sequence needs the token offsets")
     out = torch.empty((T, W), dtype=out_dtype, device=h.device)
+    slot_stride = 0                      # (a state without rows: one tap reads no row before the present one)
+    if state.shape[1] > 0:
+        slot_stride = state.stride(0) if state.shape[0] > 1 else state.shape[1] * W
     _check(_lib().llogos_causal_conv(_p(out), _DT[out_dtype], _p(h), _p(w), _p(state), _p(ctx.slots), _p(ctx.tok_seq),
                                      _p(ctx.tok_pos), _p(ctx.cu_dev), T, ctx.batch, W, h.stride(0) if T > 1 else max(W, h.stride(0)),
-                                     taps, 1 if add_input else 0, _stream()), "causal_conv")
+                                     taps, 1 if add_input else 0, _p(bias), ctypes.c_longlong(slot_stride), _stream()), "causal_conv")
     return out
 
 
@@ -768,6 +775,158 @@ def head_products(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_kn: Opt
     if T:
         _check(_lib().llogos_head_products(_p(out), _dt(out), out.stride(0), out.stride(1), _p(a), _dt(a), a.stride(0), a.stride(1),
                                            _p(w), _dt(w), T, H, N, K, _stream()), "head_products")
+    return out
+
+
+def post_norm(x: torch.Tensor, delta: Optional[torch.Tensor], alpha: float, weight: torch.Tensor, eps: float,
+              rows_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """The float32 stream x [T, H] becomes norm(alpha * x + delta) * weight in place (RMS norm, eps inside the
+    root); `delta` is [T, H] or partial sums [parts, T, H], float32 or bfloat16, or None.  With `rows_dtype`
+    the new rows are also returned in that type (for float32 that is x itself: nothing more is written)."""
+    _dev(x, weight, delta)
+    _need(x.dtype == torch.float32 and x.dim() == 2, "post_norm: x must be float32 [T, H]")
+    T, H = x.shape
+    _need(weight.dtype == torch.float32 and weight.shape == (H,), "post_norm: weight must be float32 [H]")
+    parts, part_stride = _parts(delta)
+    if delta is not None:
+        _need(tuple(delta.shape[-2:]) == (T, H), "post_norm: delta must have x's shape")
+    rows = None
+    if rows_dtype is not None and rows_dtype != torch.float32:
+        rows = torch.empty((T, H), dtype=rows_dtype, device=x.device)
+    if T:
+        _check(_lib().llogos_post_norm(_p(x), _p(delta), _dt(delta) if delta is not None else F32, parts,
+                                       ctypes.c_longlong(part_stride), ctypes.c_float(alpha), _p(weight), ctypes.c_float(eps), T, H,
+                                       _p(rows), _DT[rows.dtype] if rows is not None else F32, _stream()), "post_norm")
+    return x if (rows_dtype == torch.float32) else rows
+
+
+RECURRENCE_SEGMENT = 0       # 0: chosen by the step; > 0 forces the segment length of the gated recurrence, -1 forbids segments (tests)
+
+
+def recurrence_segments(lens: Sequence[int], channels: int, n_cus: Optional[int] = None) -> int:
+    """The segment length for a step's gated recurrences (0: every sequence whole, one thread a channel).
+    A whole sequence gives batch * channels threads, which run its tokens one after the other; segments
+    run side by side at the price of a second pass over the inputs.  They pay when the sequences are
+    long and their threads alone would leave most of the GPU idle."""
+    if RECURRENCE_SEGMENT:
+        return max(0, RECURRENCE_SEGMENT)
+    longest = max(lens)
+    if longest < 256:
+        return 0
+    n_cus = n_cus or compute_units()
+    waves = len(lens) * ((channels + 63) // 64)
+    if waves >= 8 * n_cus:
+        return 0
+    want = max(2, min(longest // 64, (8 * n_cus + waves - 1) // waves))
+    return max(64, -(-longest // want))
+
+
+def gated_recurrence(ctx, u: torch.Tensor, gates: torch.Tensor, block: int, r_bias: torch.Tensor, i_bias: torch.Tensor,
+                     decay: torch.Tensor, y: torch.Tensor, state: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """S <- a S + sqrt(1 - a^2) * (i * u) with a = exp(-decay * r), r and i the sigmoids of the gate logits;
+    returns S * gelu_tanh(y) as [T, C] in `out_dtype`.  u, y: float32 [T, C] (maybe columns of wider rows);
+    gates float32 [T, >= 2 C] laid out in blocks of `block` channels as [r logits | i logits]; r_bias, i_bias,
+    decay float32 [C]; state float32 [slots, C] (a view with its own slot stride will do): each sequence's S,
+    read at the start of its tokens and written behind them."""
+    for t_, name in ((u, "u"), (gates, "gates"), (y, "y")):
+        _need(t_.is_cuda and t_.dtype == torch.float32 and t_.dim() == 2 and t_.stride(1) == 1, f"gated_recurrence: {name} must be float32 rows on the GPU")
+    _dev(r_bias, i_bias, decay, ctx.slots, ctx.cu_dev)
+    T, C = u.shape
+    _need(T == ctx.n_tokens and y.shape == (T, C) and gates.shape[0] == T and gates.shape[1] >= 2 * C, "gated_recurrence: one row a token, 2 C gate logits")
+    _need(block > 0 and C % block == 0, "gated_recurrence: the channels must divide into the blocks")
+    for t_ in (r_bias, i_bias, decay):
+        _need(t_.dtype == torch.float32 and t_.shape == (C,), "gated_recurrence: biases and decay must be float32 [C]")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == C and state.stride(1) == 1,
+          "gated_recurrence: state must be float32 [slots, C]")
+    _need(ctx.cu_dev is not None or T == ctx.batch, "gated_recurrence: a step of several tokens a sequence needs the token offsets")
+    ld = lambda t_, least: t_.stride(0) if T > 1 else max(least, t_.stride(0))
+    out = torch.empty((T, C), dtype=out_dtype, device=u.device)
+    seg_len, n_seg, seg_first, seg_a, seg_l = 0, 0, None, None, None
+    if ctx.cu_dev is not None and not ctx.in_graph and RECURRENCE_SEGMENT >= 0:
+        lens = [ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch)]
+        seg_len = recurrence_segments(lens, C)
+        if seg_len > 0:
+            first = [0]
+            for n in lens:
+                first.append(first[-1] + -(-n // seg_len))
+            n_seg = first[-1]
+            seg_first = torch.tensor(first, dtype=torch.int32).to(u.device)
+            seg_a = torch.empty((n_seg, C), dtype=torch.float32, device=u.device)
+            seg_l = torch.empty((n_seg, C), dtype=torch.float32, device=u.device)
+    slot_stride = state.stride(0) if state.shape[0] > 1 else max(C, state.stride(0))
+    _check(_lib().llogos_gated_recurrence(
+        _p(out), _DT[out_dtype], _p(u), ld(u, C), _p(gates), ld(gates, 2 * C), int(block), _p(r_bias), _p(i_bias), _p(decay),
+        _p(y), ld(y, C), _p(state), ctypes.c_longlong(slot_stride), _p(ctx.slots), _p(ctx.cu_dev), T, ctx.batch, C,
+        int(seg_len), int(n_seg), _p(seg_first), _p(seg_a), _p(seg_l), _stream()), "gated_recurrence")
+    return out
+
+
+def rotary_prepare(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype, n_heads: int, n_kv_heads: int,
+                   dim: int, v_dim: int, maps: int, rot: int, pairing: int, cs: Optional[torch.Tensor],
+                   q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], unit_after: bool, eps: float,
+                   k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor], table: Optional[torch.Tensor],
+                   writes: bool = True) -> torch.Tensor:
+    """From projected rows [q | k | v] ([T, >= W] or partial sums [parts, T, >= W], float32 or the cache's type,
+    plus `bias` [W]; W = (n_heads + n_kv_heads) * maps * dim + n_kv_heads * v_dim): every run of `dim` values of q
+    and k (a head, or one of a head's `maps` score maps) gets an RMS norm with a shared weight where one is given,
+    then the rotation of its first `rot` dimensions by the table `cs` [T, rot / 2, 2], then, with `unit_after`,
+    is divided by its root mean square.  q comes back [T, n_heads * maps * dim] in `out_dtype`; a kv head's `maps`
+    key runs go side by side into its key page row, its v_dim values into its value page row.  writes False:
+    only q is made."""
+    _need(qkv.is_cuda and qkv.stride(-1) == 1 and (qkv.dtype == torch.float32 or qkv.dtype == out_dtype),
+          "rotary_prepare: rows must be float32 or the cache's type, on the GPU")
+    _dev(bias, q_norm_w, k_norm_w, cs, table, ctx.tok_seq, ctx.tok_pos)
+    parts, part_stride = _parts(qkv)
+    T = qkv.shape[-2]
+    Wq, Wk, Wv = n_heads * maps * dim, n_kv_heads * maps * dim, n_kv_heads * v_dim
+    width = Wq + ((Wk + Wv) if writes else 0)
+    _need(qkv.shape[-1] >= width and T == ctx.n_tokens, f"rotary_prepare: rows of at least {width} values, one a token")
+    _need(maps >= 1 and 0 < dim <= GENERIC_MAX_HEAD_DIM and 0 < v_dim <= GENERIC_MAX_HEAD_DIM, "rotary_prepare: head sizes out of range")
+    _need(rot % 2 == 0 and 0 <= rot <= dim and pairing in (0, 1), "rotary_prepare: the rotated width must be even and within a run")
+    if rot:
+        _need(cs is not None and cs.dtype == torch.float32 and tuple(cs.shape) == (T, rot // 2, 2), "rotary_prepare: rotary table shape")
+    row_stride = qkv.stride(-2) if T > 1 else max(Wq + Wk + Wv, qkv.stride(-2))
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() >= width, f"rotary_prepare: bias must be float32 [{width}]")
+    for wgt in (q_norm_w, k_norm_w):
+        if wgt is not None:
+            _need(wgt.dtype == torch.float32 and wgt.shape == (dim,), "rotary_prepare: a norm weight must be float32 [dim]")
+    kd = vd = 0
+    if writes:
+        _need(k_pool is not None and v_pool is not None and table is not None, "rotary_prepare: cache missing")
+        _i32(table, "table")
+        _need(k_pool.dtype == out_dtype and v_pool.dtype == out_dtype, "rotary_prepare: cache type differs")
+        kd, vd = _page_dims(k_pool, v_pool, n_kv_heads, "rotary_prepare")
+        _need(kd >= maps * dim and vd >= v_dim and table.dim() == 2, "rotary_prepare: pages narrower than the heads")
+    q_out = torch.empty((T, Wq), dtype=out_dtype, device=qkv.device)
+    _check(_lib().llogos_rotary_prepare(
+        _p(qkv), _dt(qkv), parts, ctypes.c_longlong(part_stride), row_stride, _p(bias), _p(q_out), _DT[out_dtype], n_heads * maps,
+        n_kv_heads if writes else 0, dim, v_dim, maps, rot, pairing, _p(q_norm_w), _p(k_norm_w), 1 if unit_after else 0,
+        ctypes.c_float(eps), _p(cs), _p(k_pool) if writes else None, _p(v_pool) if writes else None, kd, vd,
+        _p(table) if writes else None, table.stride(0) if (writes and table is not None) else 0, _p(ctx.tok_seq), _p(ctx.tok_pos),
+        T, _stream()), "rotary_prepare")
+    return q_out
+
+
+def diff_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor, n_heads: int,
+                   n_kv_heads: int, dim: int, v_dim: int, scale: float, lam: float, out_scale: float, eps: float,
+                   window: int = 0, sinks: int = 0) -> torch.Tensor:
+    """Differential attention of the step's query rows q [T, n_heads * 2 * dim] (head by head [map 1 | map 2]) over
+    their sequences' pages, whose key rows hold both maps' keys side by side: two softmax maps over the same
+    values, out = (a_1 - lam * a_2) / rms(a_1 - lam * a_2) * out_scale per head.  Returns [T, n_heads * v_dim]."""
+    T = ctx.n_tokens
+    _dev(q, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos)
+    _i32(table, "table")
+    _need(q.dtype == k_pool.dtype and tuple(q.shape) == (T, n_heads * 2 * dim), "diff_attention: q must be [T, heads * 2 * dim] of the cache's type")
+    _need(n_heads % n_kv_heads == 0, "diff_attention: heads must be a multiple of kv heads")
+    kd, vd = _page_dims(k_pool, v_pool, n_kv_heads, "diff_attention")
+    _need(v_pool is not None and kd >= 2 * dim and vd >= v_dim, "diff_attention: pages narrower than the heads")
+    _need(2 * dim <= GENERIC_MAX_HEAD_DIM and 0 < v_dim <= GENERIC_MAX_HEAD_DIM, "diff_attention: head sizes out of range")
+    out = torch.empty((T, n_heads * v_dim), dtype=q.dtype, device=q.device)
+    _check(_lib().llogos_diff_attention_generic(
+        _p(out), _p(q), _dt(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(ctx.tok_seq), _p(ctx.tok_pos),
+        T, n_heads, n_kv_heads, dim, v_dim, kd, vd, ctypes.c_float(scale), int(window), int(sinks), ctypes.c_float(lam),
+        ctypes.c_float(out_scale), ctypes.c_float(eps), _stream()), "diff_attention")
     return out
 
 

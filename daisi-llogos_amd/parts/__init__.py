@@ -13,4 +13,6 @@ from .mlp import ActivatedMLP, SwiGLU
 from .capped_attention import CappedAttention
 from .moe import TableMoE
 from .loop import LoopEntry
-from .block import ParallelBlock, PreNormBlock, SandwichBlock
+from .rglru import RGLRU
+from .diff_attention import DiffAttention
+from .block import ParallelBlock, PostNormBlock, PreNormBlock, SandwichBlock

@@ -222,3 +222,77 @@ class ParallelBlock(Block):
             d = self.ffn.forward(ctx, h)
         mark(ctx, "feed_forward")
         return x, d
+
+
+@register_block("post_norm")
+class PostNormBlock(Block):
+    """The norm comes after the residual sum, and the stream itself is what the sublayers read:
+
+        x <- mixer_norm(alpha * x + mixer(x));   x <- ffn_norm(alpha * x + ffn(x))
+
+    The feed-forward (with its norm) may be absent.  The stream stays float32; each closing kernel
+    (ops.kernels.post_norm: scaled sum, norm, weight) also leaves the new rows in the runtime's type for the
+    sublayer that reads them next, and the block hands the last such rows on in place of a delta
+    (`NormedAhead(rows, None)`: the stream is complete, and these are its own rows), which a block of this
+    kind takes up and every norm ignores.  Norms that are not RMS norms with a row weight run their own
+    kernel on the scaled sum instead."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None,
+                 alpha: float = 1.0):
+        if ffn is not None and ffn_norm is None:
+            raise ValueError("a feed-forward comes with the norm behind its sum")
+        # (a second norm without a feed-forward norms the scaled stream alone)
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+        self.alpha = float(alpha)
+
+    def mixers(self) -> List[Mixer]:
+        return [self.mixer]
+
+    def feed_forwards(self) -> List[FeedForward]:
+        return [self.ffn] if self.ffn is not None else []
+
+    def parts(self) -> List[Part]:
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def entry_norm(self) -> Optional[Norm]:
+        return None                      # the block's first reader takes the stream as it is
+
+    def _close(self, x: torch.Tensor, out, norm: Norm) -> torch.Tensor:
+        """x <- norm(alpha * x + out) in place; returns the new rows in the runtime's type."""
+        from ..ops import kernels as K
+        w = norm.row_weight()
+        if w is not None and (out is None or isinstance(out, torch.Tensor)):
+            return K.post_norm(x, out, self.alpha, w, norm.eps, self.rt.dtype)
+        # any other norm: the stream scaled by a plain kernel, then the norm's own kernel, which adds `out`
+        # (float32 rows where the norm can make them; a norm of the plain interface gives the runtime's type)
+        import inspect
+        K.scale_softcap(x, self.alpha)
+        if "out_dtype" in inspect.signature(norm.forward).parameters:
+            rows = norm.forward(x, out, out_dtype=torch.float32)
+        else:
+            rows = norm.forward(x, out)
+        x.copy_(rows)
+        return x if self.rt.is_f32 else K.sum_parts(x, None, self.rt.dtype)
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches):
+        from ..ops import kernels as K
+        cache = caches[0] if isinstance(caches, (list, tuple)) else caches
+        if isinstance(pending, NormedAhead) and pending.norm is None and pending.rows.dtype == self.rt.dtype:
+            h = pending.rows                                  # the block before left the stream's rows
+        else:
+            if isinstance(pending, torch.Tensor):
+                K.residual_add(x, K.sum_parts(pending, None, torch.float32))
+            h = x if self.rt.is_f32 else K.sum_parts(x, None, self.rt.dtype)
+        mark(ctx, "norm")
+        a = self.mixer.forward(ctx, h, cache)
+        mark(ctx, "mixer")
+        h = self._close(x, a, self.mixer_norm)
+        mark(ctx, "norm")
+        if self.ffn_norm is not None:
+            d = None
+            if self.ffn is not None:
+                d = self.ffn.forward(ctx, h)
+                mark(ctx, "feed_forward")
+            h = self._close(x, d, self.ffn_norm)
+            mark(ctx, "norm")
+        return x, (None if self.rt.is_f32 else NormedAhead(h, None))
