@@ -175,6 +175,26 @@ def zogurax_config(width, runs, vocab, ff):
             "torch_dtype": "bfloat16"}
 
 
+def batodra_config(width, layers, vocab, ff):
+    """Layers of real sizes: a gated linear recurrence, window attention, a recurrence and differential attention in
+    turn, a feed-forward behind each; recurrences as wide as the stream with blocks of 256 channels and four taps;
+    window attention with heads of 128 dimensions, four query heads a key/value head, a window of 1,024 tokens that
+    keeps the first four; differential attention with two maps of 64 dimensions and values of 128 a head."""
+    heads = width // 128
+    kv = max(1, heads // 4)
+    mlp = {"kind": "dense", "ff": ff}
+    rec = {"type": "rglru", "mixer": {"width": width, "blocks": max(1, width // 256), "conv": 4}, "mlp": mlp}
+    win = {"type": "attention_2",
+           "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 0.125, "mask": {"size": 1024, "keep_first": 4},
+                     "rot": {"base": 500000.0, "dims": 128, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+           "mlp": mlp}
+    dif = {"type": "attention",
+           "mixer": {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.5, "rot": {"base": 500000.0, "dims": 64}},
+           "mlp": mlp}
+    return {"architecture": "Batodra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 2.0,
+            "layers": [(rec, win, rec, dif)[i % 4] for i in range(layers)], "torch_dtype": "bfloat16"}
+
+
 def moe_bytes_read(model, ids) -> int:
     """Bytes of weights that a step with the token ids `ids` reads: as step_weight_bytes, but of a layer's experts
     only those that the layer's table names for these ids."""
@@ -261,6 +281,8 @@ def compare_designs(args) -> int:
                      num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), tie_word_embeddings=True)
         if args.design == "zogurax":
             other = zogurax_config(width, layers, vocab, ff)
+        elif args.design == "batodra":
+            other = batodra_config(width, layers, vocab, ff * 3 // 2)
         else:
             # two matrices a feed-forward instead of three: half as wide again for the same weight
             other = nipulorn_config(width, layers, vocab, ff * 3 // 2)
@@ -272,7 +294,7 @@ def compare_designs(args) -> int:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["nipulorn", "zogurax"], default=None,
+    ap.add_argument("--design", choices=["nipulorn", "zogurax", "batodra"], default=None,
                     help="instead of the default run: this design beside the dense decoder at equal sizes (prefill, decode, parts)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=248)   # + 8 warm-up = 256 new tokens

@@ -327,7 +327,11 @@ struct DirectPageLds {
 // VD: the values' width where it is not the keys' (HD); BENT: the scores are scaled and bent through a tanh before
 // the softmax (cap > 0), a row may end with a sink of score 0 in its denominator (unit_sink) and with a gate on its
 // head (gate [tokens, gate_stride] logits), and there is no window.
-template <int HD, int HALVES, int VD = HD, bool BENT = false>
+// MAPS = 2: every head has two score maps over the same values (differential attention).  A map is a head of its own
+// here: the caller gives twice the heads and twice the group, head 2 h + m is map m of head h; a kv head's key row
+// in its page holds the maps' keys side by side (MAPS * HD values), of which a block copies its own map's; and the
+// rows come out as 32-bit floats [tokens][heads][maps][VD] for the kernel that takes the maps' difference.
+template <int HD, int HALVES, int VD = HD, bool BENT = false, int MAPS = 1>
 __global__ __launch_bounds__(HALVES * kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_prefill_direct_kernel(
         bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
@@ -404,12 +408,15 @@ void attn_prefill_direct_kernel(
     // This wave's share of a page's copy, in instructions of 1 KB (64 lanes x 16 bytes, a fragment):
     // the block's instructions go to its waves in turn.
     auto copy_page = [&](int id, DirectPageLds<HD, VD>& pg) {
-        const bf16_t* kpage = k_pool + page_base(id) * HD;
+        const bf16_t* kpage = k_pool + page_base(id) * (MAPS * HD);
         const bf16_t* vpage = v_pool + page_base(id) * VD;
 #pragma unroll
-        for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
+        for (int j = 0; j < (HD / 8 + kAttnWaves - 1) / kAttnWaves; ++j) {
             const int f = kAttnWaves * j + wave;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kpage + 512 * f + 8 * lane),
+            if ((HD / 8) % kAttnWaves != 0 && f >= HD / 8) break;        // (the same for a whole wave)
+            // fragment (rb, sk) of this map within the row of all maps' keys
+            const int src = MAPS == 1 ? f : (f / (HD / 32)) * (MAPS * HD / 32) + (h % MAPS) * (HD / 32) + f % (HD / 32);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kpage + 512 * src + 8 * lane),
                                              (__attribute__((address_space(3))) void*)&pg.k[f][0], 16, 0, 0);
         }
 #pragma unroll
@@ -576,6 +583,14 @@ void attn_prefill_direct_kernel(
         if (rr >= wave_rows) return;
         const float inv = BENT ? finish_factor(st.m, st.l, unit_sink, gate ? gate + (size_t)(row0 + rr) * gate_stride + h : nullptr)
                                : (st.l > 0.f ? 1.0f / st.l : 0.f);
+        if (MAPS > 1) {
+            float* frow = reinterpret_cast<float*>(out) + ((size_t)(row0 + rr) * n_heads + h) * VD;
+#pragma unroll
+            for (int db = 0; db < VD / 16; ++db)
+                *reinterpret_cast<f32x4*>(frow + 16 * db + 4 * g) = f32x4{st.acc[db][0] * inv, st.acc[db][1] * inv,
+                                                                          st.acc[db][2] * inv, st.acc[db][3] * inv};
+            return;
+        }
         bf16_t* orow = out + ((size_t)(row0 + rr) * n_heads + h) * VD;
 #pragma unroll
         for (int db = 0; db < VD / 16; ++db) {

@@ -908,6 +908,10 @@ def rotary_prepare(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dty
     return q_out
 
 
+DIFF_MFMA = True             # False keeps differential attention off the matrix cores (tests)
+DIFF_PREFILL_HALVES = 0      # 0: chosen by the step; 1 or 2 forces the sets of waves a block of its prompt kernel (tests)
+
+
 def diff_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor, n_heads: int,
                    n_kv_heads: int, dim: int, v_dim: int, scale: float, lam: float, out_scale: float, eps: float,
                    window: int = 0, sinks: int = 0) -> torch.Tensor:
@@ -923,10 +927,36 @@ def diff_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Ten
     _need(v_pool is not None and kd >= 2 * dim and vd >= v_dim, "diff_attention: pages narrower than the heads")
     _need(2 * dim <= GENERIC_MAX_HEAD_DIM and 0 < v_dim <= GENERIC_MAX_HEAD_DIM, "diff_attention: head sizes out of range")
     out = torch.empty((T, n_heads * v_dim), dtype=q.dtype, device=q.device)
+    if q.dtype == torch.bfloat16 and DIFF_MFMA and q.is_contiguous() and kd == 2 * dim and vd == v_dim:
+        # head shapes the matrix-core kernels take run there; -2 says that this one is none of them
+        lib = _lib()
+        if ctx.is_decode:
+            width = table.shape[1]
+            _need(table.shape[0] == T and ctx.tok_pos.numel() == T, "diff_attention: one table row and position a sequence")
+            ws = _attn_workspace(q.device, lib.llogos_diff_attn_decode_workspace(T, n_heads, n_kv_heads, v_dim, width))
+            code = lib.llogos_diff_attn_decode_bf16(
+                _p(out), _p(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), width, _p(ctx.tok_pos), T,
+                n_heads, n_kv_heads, dim, v_dim, ctypes.c_float(scale), int(window), int(sinks), ctypes.c_float(lam),
+                ctypes.c_float(out_scale), ctypes.c_float(eps), _p(ws), ctypes.c_longlong(ws.numel()), _stream())
+        else:
+            cu = ctx.cu_dev
+            _need(cu is not None and cu.numel() == ctx.batch + 1, "diff_attention: the step's token offsets are missing")
+            lens = [ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch)]
+            n_tiles = sum(-(-n // 128) for n in lens)
+            halves = DIFF_PREFILL_HALVES or prefill_halves(lens, getattr(ctx, "starts", None), 2 * n_heads)
+            ws = torch.empty(lib.llogos_diff_attn_prefill_workspace(T, n_heads, v_dim), dtype=torch.float32, device=q.device)
+            code = lib.llogos_diff_attn_prefill_bf16(
+                _p(out), _p(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
+                ctx.batch, T, n_tiles, n_heads, n_kv_heads, dim, v_dim, ctypes.c_float(scale), int(window), int(sinks),
+                ctypes.c_float(lam), ctypes.c_float(out_scale), ctypes.c_float(eps), int(halves), _p(ws),
+                ctypes.c_longlong(ws.numel()), _stream())
+        if code != -2:
+            _check(code, "diff_attention")
+            return out
     _check(_lib().llogos_diff_attention_generic(
         _p(out), _p(q), _dt(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(ctx.tok_seq), _p(ctx.tok_pos),
         T, n_heads, n_kv_heads, dim, v_dim, kd, vd, ctypes.c_float(scale), int(window), int(sinks), ctypes.c_float(lam),
-        ctypes.c_float(out_scale), ctypes.c_float(eps), _stream()), "diff_attention")
+        ctypes.c_float(out_scale), ctypes.c_float(eps), _stream()), "diff_attention_generic")
     return out
 
 

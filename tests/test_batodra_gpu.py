@@ -200,10 +200,18 @@ DIFFERENTIAL = [(6, 2, 16, 24, 56, 16), (2, 2, 64, 128, 64, 32), (1, 1, 8, 40, 4
                 (4, 2, 64, 64, 64, 64), (8, 2, 32, 32, 64, 16), (2, 1, 128, 128, 96, 64)]
 
 
-def _differential(heads, kv, d, dv, hidden, rot, diff=0.3, scale=0.5, base=100.0):
+def _differential(heads, kv, d, dv, hidden, rot, diff=0.3, scale=0.5, base=100.0, window=0, keep=0):
     position = P.Rotary(d, rot, base) if rot else None
     return P.DiffAttention(prefix="m.", hidden=hidden, n_heads=heads, n_kv_heads=kv, head_dim=d, v_dim=dv, scale=scale, diff=diff,
-                           position=position, eps=1e-5)
+                           position=position, eps=1e-5, window=window, sinks=keep)
+
+
+def _on_the_matrix_cores(monkeypatch, d, dv):
+    """Shapes that the matrix-core kernels take must run there in bfloat16."""
+    if d in (32, 64, 128) and dv in (64, 128):
+        check = K._check
+        monkeypatch.setattr(K, "_check", lambda code, name: pytest.fail("the kernel for any shape ran") if name == "diff_attention_generic"
+                            else check(code, name))
 
 
 def _plain_differential(mix, plain, h, rot, base=100.0):
@@ -212,10 +220,13 @@ def _plain_differential(mix, plain, h, rot, base=100.0):
     return pb.differential_attention(m, plain, "m.", h, np.arange(len(h)), mix.eps)
 
 
-@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("dtype,halves", [("float32", 0), ("bfloat16", 0), ("bfloat16", 1), ("bfloat16", 2)])
 @pytest.mark.parametrize("shape", DIFFERENTIAL)
-def test_differential_attention_alone_in_pieces(shape, dtype):
+def test_differential_attention_alone_in_pieces(shape, dtype, halves, monkeypatch):
     heads, kv, d, dv, hidden, rot = shape
+    monkeypatch.setattr(K, "DIFF_PREFILL_HALVES", halves)            # either form of the prompt kernel in turn
+    if dtype == "bfloat16":
+        _on_the_matrix_cores(monkeypatch, d, dv)
     rng = np.random.default_rng(heads * 100 + d)
     mix = _differential(*shape)
     plain = _bind(mix, rng, dtype, scaled={"m.lq1": 2.0, "m.lk2": 2.0})
@@ -227,11 +238,31 @@ def test_differential_attention_alone_in_pieces(shape, dtype):
         assert np.abs(g - w_).max() <= (2 if dtype == "bfloat16" else 1) * PART_TOL[dtype] * max(1.0, np.abs(w_).max()), f"sequence {i}"
 
 
-def test_a_far_key_decides_in_each_map_of_differential_attention():
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("shape", [(4, 2, 64, 64, 64, 64), (6, 2, 16, 24, 56, 16)])
+def test_differential_attention_behind_a_window_that_keeps_the_first_tokens(shape, dtype, monkeypatch):
+    """The mixer takes a window like the plain attention does (the design's own layers give it none)."""
+    heads, kv, d, dv, hidden, rot = shape
+    if dtype == "bfloat16":
+        _on_the_matrix_cores(monkeypatch, d, dv)
+    rng = np.random.default_rng(d)
+    mix = _differential(*shape, window=70, keep=3)
+    plain = _bind(mix, rng, dtype)
+    h = _inputs(rng, hidden, dtype)
+    sees = pb.visible
+    monkeypatch.setattr(pb, "visible", lambda p, window=0, keep_first=0: sees(p, 70, 3))
+    want = [_plain_differential(mix, plain, x, rot) for x in h]
+    got = _pieces(mix, dtype, h, LENGTHS, CUTS, PAGES, SLOTS)
+    for i, (g, w_) in enumerate(zip(got, want)):
+        assert np.abs(g - w_).max() <= (2 if dtype == "bfloat16" else 1) * PART_TOL[dtype] * max(1.0, np.abs(w_).max()), f"sequence {i}"
+
+
+@pytest.mark.parametrize("dv", [48, 64])
+def test_a_far_key_decides_in_each_map_of_differential_attention(dv):
     """The query matrix of one map is the key matrix with its columns reversed, and the late tokens are an early
     token reversed: their queries point at that token's key in that map alone, so it outweighs hundreds of others.
     Without that key the plain result moves by many times the bound, for either map; the kernels agree with it there."""
-    heads, kv, d, dv, hidden, rot = 4, 2, 32, 48, 64, 8
+    heads, kv, d, hidden, rot = 4, 2, 32, 64, 8
     for which in (0, 1):
         rng = np.random.default_rng(7 + which)
         mix = _differential(heads, kv, d, dv, hidden, rot, scale=1.0, base=50000.0)
