@@ -286,8 +286,12 @@ def compare_designs(args) -> int:
         else:
             # two matrices a feed-forward instead of three: half as wide again for the same weight
             other = nipulorn_config(width, layers, vocab, ff * 3 // 2)
-        record["sizes"].append({"size": name, "layers": layers, args.design: measure(f"{args.design} {name}", other, vocab),
-                                "dense": measure(f"dense {name}", dense, vocab)})
+        entry = {"size": name, "layers": layers, args.design: measure(f"{args.design} {name}", other, vocab)}
+        if args.design == "batodra":
+            # the other design that mixes recurrent layers with attention, at the same sizes
+            entry["nipulorn"] = measure(f"nipulorn {name}", nipulorn_config(width, layers, vocab, ff * 3 // 2), vocab)
+        entry["dense"] = measure(f"dense {name}", dense, vocab)
+        record["sizes"].append(entry)
     print(json.dumps(record), flush=True)
     return 0
 

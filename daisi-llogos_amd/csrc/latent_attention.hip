@@ -160,12 +160,13 @@ __global__ __launch_bounds__(256) void head_products_few_kernel(TO* __restrict__
     // this thread: output n, the k of its group: kg, kg + 4, ... (the groups' loads of w lie 4 rows apart)
     if (n < N) {
         const TW* wp = w_kn + (size_t)h * K * N + n;
-        for (int k0 = kg; k0 < K; k0 += 16) {
-            float wv[4];
+        // (sixteen loads in flight: a thread's loads are 2 or 4 bytes each, and their latency is what the kernel waits for)
+        for (int k0 = kg; k0 < K; k0 += 64) {
+            float wv[16];
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) wv[kk] = k0 + 4 * kk < K ? load_f32(wp + (size_t)(k0 + 4 * kk) * N) : 0.f;
+            for (int kk = 0; kk < 16; ++kk) wv[kk] = k0 + 4 * kk < K ? load_f32(wp + (size_t)(k0 + 4 * kk) * N) : 0.f;
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
+            for (int kk = 0; kk < 16; ++kk) {
                 const int k = min(k0 + 4 * kk, K - 1);                   // (beyond the end: wv is 0)
 #pragma unroll
                 for (int t = 0; t < TMAX; ++t) acc[t] = fmaf(rows_lds[k * TMAX + t], wv[kk], acc[t]);

@@ -8,7 +8,14 @@
 template <typename TD>
 __device__ __forceinline__ float pn_sum_parts(const TD* p, size_t i, int parts, size_t part_stride) {
     float v = load_f32(p + i);
-    for (int q = 1; q < parts; ++q) v += load_f32(p + q * part_stride + i);
+    for (int q0 = 1; q0 < parts; q0 += 8) {          // eight loads in flight, added in ascending order
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = q0 + j < parts ? load_f32(p + (size_t)(q0 + j) * part_stride + i) : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (q0 + j < parts) v += y[j];
+    }
     return v;
 }
 
