@@ -136,15 +136,15 @@ __global__ __launch_bounds__(256) void head_products_kernel(TO* __restrict__ out
 }
 
 // The same for steps of up to 16 rows, where the tiles above would be nearly empty: the rows of a head go to
-// LDS once, a thread owns an output n and a quarter of k and streams its part of the head's matrix, which for
-// this kernel is stored k-major, w_kn [H, K, N], so that neighbouring threads read neighbouring values; the four
-// quarters are added in a fixed order.  TMAX: the rows
+// LDS once, a thread owns an output n and one of KG groups of k and streams its part of the head's matrix, which for
+// this kernel is stored k-major, w_kn [H, K, N], so that neighbouring threads read neighbouring values; the
+// groups' sums are added in a fixed order.  TMAX: the rows
 // rounded up to 1, 2, 4, 8 or 16 (rows that are not there are zeros in LDS).
-template <int TMAX, typename TA, typename TW, typename TO>
-__global__ __launch_bounds__(256) void head_products_few_kernel(TO* __restrict__ out, int ldo, int o_head, const TA* __restrict__ a, int lda, int a_head,
+template <int TMAX, int KG, typename TA, typename TW, typename TO>
+__global__ __launch_bounds__(64 * KG) void head_products_few_kernel(TO* __restrict__ out, int ldo, int o_head, const TA* __restrict__ a, int lda, int a_head,
                                          const TW* __restrict__ w_kn, int M, int N, int K) {
-    // LDS: the head's rows as [k][TMAX] (one or two 16-byte reads bring every row's value of a k), then the four
-    // k-groups' sums [4][64][TMAX]
+    // LDS: the head's rows as [k][TMAX] (one or two 16-byte reads bring every row's value of a k), then the KG
+    // k-groups' sums [KG][64][TMAX]
     extern __shared__ float rows_lds[];
     float* sums = rows_lds + (size_t)K * TMAX;
     const int h = blockIdx.y, nl = threadIdx.x & 63, kg = threadIdx.x >> 6, n = blockIdx.x * 64 + nl;
@@ -157,17 +157,18 @@ __global__ __launch_bounds__(256) void head_products_few_kernel(TO* __restrict__
     float acc[TMAX];
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) acc[t] = 0.f;
-    // this thread: output n, the k of its group: kg, kg + 4, ... (the groups' loads of w lie 4 rows apart)
+    // this thread: output n, the k of its group: kg, kg + KG, ... (the groups' loads of w lie KG rows apart)
     if (n < N) {
         const TW* wp = w_kn + (size_t)h * K * N + n;
-        // (sixteen loads in flight: a thread's loads are 2 or 4 bytes each, and their latency is what the kernel waits for)
-        for (int k0 = kg; k0 < K; k0 += 64) {
+        // (sixteen loads in flight: a thread's loads are 2 or 4 bytes each, and their latency is what the kernel waits for;
+        // sixteen groups of k give a compute unit's SIMDs four waves each to wait with)
+        for (int k0 = kg; k0 < K; k0 += 16 * KG) {
             float wv[16];
 #pragma unroll
-            for (int kk = 0; kk < 16; ++kk) wv[kk] = k0 + 4 * kk < K ? load_f32(wp + (size_t)(k0 + 4 * kk) * N) : 0.f;
+            for (int kk = 0; kk < 16; ++kk) wv[kk] = k0 + KG * kk < K ? load_f32(wp + (size_t)(k0 + KG * kk) * N) : 0.f;
 #pragma unroll
             for (int kk = 0; kk < 16; ++kk) {
-                const int k = min(k0 + 4 * kk, K - 1);                   // (beyond the end: wv is 0)
+                const int k = min(k0 + KG * kk, K - 1);                  // (beyond the end: wv is 0)
 #pragma unroll
                 for (int t = 0; t < TMAX; ++t) acc[t] = fmaf(rows_lds[k * TMAX + t], wv[kk], acc[t]);
             }
@@ -179,7 +180,9 @@ __global__ __launch_bounds__(256) void head_products_few_kernel(TO* __restrict__
     if (kg == 0 && n < N) {
 #pragma unroll
         for (int t = 0; t < TMAX; ++t) {
-            const float v = ((sums[(0 * 64 + nl) * TMAX + t] + sums[(1 * 64 + nl) * TMAX + t]) + sums[(2 * 64 + nl) * TMAX + t]) + sums[(3 * 64 + nl) * TMAX + t];
+            float v = sums[nl * TMAX + t];
+#pragma unroll
+            for (int j = 1; j < KG; ++j) v += sums[(j * 64 + nl) * TMAX + t];          // in the groups' order
             if (t < M) store_f32(out + (size_t)t * ldo + (size_t)h * o_head + n, v);
         }
     }
@@ -191,12 +194,25 @@ LLOGOS_EXPORT int llogos_head_products_few(void* out, int out_dtype, int ldo, in
     if (M <= 0 || M > 16 || H <= 0 || N <= 0 || K <= 0) return LLOGOS_BAD_ARGUMENT;
     int tmax = 1;
     while (tmax < M) tmax <<= 1;
-    const size_t smem = (size_t)tmax * (K + 256) * sizeof(float);
+    // sixteen groups of k where their sums fit beside the rows and every group has k of its own, else four
+    const bool wide = K >= 64 && (size_t)tmax * (K + 16 * 64) * sizeof(float) <= 65536;
+    const size_t smem = (size_t)tmax * (K + (wide ? 16 : 4) * 64) * sizeof(float);
     if (smem > 65536) return LLOGOS_UNSUPPORTED;
-    const int threads = 256;
     dim3 grid((N + 63) / 64, H);
-#define HPF(TM, TA, TW, TO) head_products_few_kernel<TM, TA, TW, TO><<<grid, threads, smem, stream>>>((TO*)out, ldo, o_head, \
-        (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K)
+#define HPF(TM, TA, TW, TO) do { \
+        if (wide) { \
+            if (smem > 48 * 1024) { \
+                hipError_t e = hipFuncSetAttribute((const void*)head_products_few_kernel<TM, 16, TA, TW, TO>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+                if (e != hipSuccess) return (int)e; \
+            } \
+            head_products_few_kernel<TM, 16, TA, TW, TO><<<grid, 1024, smem, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K); \
+        } else { \
+            if (smem > 48 * 1024) { \
+                hipError_t e = hipFuncSetAttribute((const void*)head_products_few_kernel<TM, 4, TA, TW, TO>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+                if (e != hipSuccess) return (int)e; \
+            } \
+            head_products_few_kernel<TM, 4, TA, TW, TO><<<grid, 256, smem, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K); \
+        } } while (0)
 #define HPT(TA, TW, TO) do { if (tmax == 1) HPF(1, TA, TW, TO); else if (tmax == 2) HPF(2, TA, TW, TO); else if (tmax == 4) HPF(4, TA, TW, TO); \
                              else if (tmax == 8) HPF(8, TA, TW, TO); else HPF(16, TA, TW, TO); } while (0)
     if (a_dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32) HPT(float, float, float);

@@ -17,11 +17,19 @@ constexpr int kPrepMaxDim = 1024;
 template <typename TI>
 __device__ __forceinline__ float rp_sum_parts(const TI* p, size_t i, int parts, size_t part_stride) {
     float v = load_f32(p + i);
-    for (int q = 1; q < parts; ++q) v += load_f32(p + q * part_stride + i);
+    for (int q0 = 1; q0 < parts; q0 += 8) {          // eight loads in flight, added in ascending order
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = q0 + j < parts ? load_f32(p + (size_t)(q0 + j) * part_stride + i) : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (q0 + j < parts) v += y[j];
+    }
     return v;
 }
 
-template <typename TI, typename T>
+// R: values a lane holds of a unit (dim <= 64 R).
+template <typename TI, typename T, int R>
 __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, size_t part_stride, int row_stride,
                                       const float* __restrict__ bias, T* __restrict__ q_out, int n_q, int n_k, int n_v,
                                       int dim, int v_dim, int maps, int rot, int pairing,
@@ -71,10 +79,10 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
     const int half = rot / 2;
     const float2* c = cs + (size_t)t * half;
     // a lane's rotated values: dimensions lane, lane + 64, ... (both partners are read before either is stored)
-    float mine[kPrepMaxDim / kWave];
+    float mine[R];
     float s2 = 0.f;
 #pragma unroll
-    for (int r = 0; r < kPrepMaxDim / kWave; ++r) {
+    for (int r = 0; r < R; ++r) {
         const int d = lane + r * kWave;
         float v = 0.f;
         if (d < dim) {
@@ -98,7 +106,7 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
     if (is_q) {
         T* dst = q_out + ((size_t)t * n_q + unit) * dim;
 #pragma unroll
-        for (int r = 0; r < kPrepMaxDim / kWave; ++r) {
+        for (int r = 0; r < R; ++r) {
             const int d = lane + r * kWave;
             if (d < dim) store_f32(dst + d, mine[r] * after);
         }
@@ -107,7 +115,7 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
         T* dst = k_pool + paged_base(cache, tok_seq[t], ku / maps, pos);
         const int col = (ku % maps) * dim;
 #pragma unroll
-        for (int r = 0; r < kPrepMaxDim / kWave; ++r) {
+        for (int r = 0; r < R; ++r) {
             const int d = lane + r * kWave;
             if (d < dim) store_f32(dst + page_key_offset(in_page, col + d, cache.head_dim), mine[r] * after);
         }
@@ -133,13 +141,16 @@ LLOGOS_EXPORT int llogos_rotary_prepare(const void* qkv, int in_dtype, int parts
     const int lds_row = dim > v_dim ? dim : v_dim;
     dim3 grid(T, (units + kPrepUnitsPerBlock - 1) / kPrepUnitsPerBlock), block(kWave, kPrepUnitsPerBlock);
     const size_t smem = (size_t)kPrepUnitsPerBlock * lds_row * sizeof(float);
-#define LAUNCH(TI, T_) rotary_prepare_kernel<TI, T_><<<grid, block, smem, stream>>>( \
+#define LAUNCH_R(TI, T_, R_) rotary_prepare_kernel<TI, T_, R_><<<grid, block, smem, stream>>>( \
         (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_q, n_k, n_v, dim, v_dim, maps, rot, pairing, \
         q_norm_w, k_norm_w, unit_after, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, v_page_dim, tok_seq, tok_pos, lds_row)
+#define LAUNCH(TI, T_) do { if (dim <= kWave) LAUNCH_R(TI, T_, 1); else if (dim <= 2 * kWave) LAUNCH_R(TI, T_, 2); \
+        else if (dim <= 4 * kWave) LAUNCH_R(TI, T_, 4); else LAUNCH_R(TI, T_, kPrepMaxDim / kWave); } while (0)
     if (dtype == DT_F32 && in_dtype == DT_F32) LAUNCH(float, float);
     else if (dtype == DT_BF16 && in_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
     else if (dtype == DT_BF16 && in_dtype == DT_F32) LAUNCH(float, bf16_t);
     else return LLOGOS_BAD_ARGUMENT;
 #undef LAUNCH
+#undef LAUNCH_R
     return LLOGOS_LAUNCH_CHECK();
 }

@@ -850,7 +850,15 @@ def gated_recurrence(ctx, u: torch.Tensor, gates: torch.Tensor, block: int, r_bi
             for n in lens:
                 first.append(first[-1] + -(-n // seg_len))
             n_seg = first[-1]
-            seg_first = torch.tensor(first, dtype=torch.int32).to(u.device)
+            # the segments' offsets, made on the device from the step's token offsets (a copy from the host would
+            # wait for the stream to drain), once a step for every layer that cuts it alike
+            key = ("recurrence_segments", seg_len)
+            seg_first = ctx.shared.get(key)
+            if seg_first is None:
+                counts = (ctx.cu_dev[1:] - ctx.cu_dev[:-1] + (seg_len - 1)) // seg_len
+                seg_first = torch.zeros(ctx.batch + 1, dtype=torch.int32, device=u.device)
+                seg_first[1:] = torch.cumsum(counts, 0)
+                ctx.shared[key] = seg_first
             seg_a = torch.empty((n_seg, C), dtype=torch.float32, device=u.device)
             seg_l = torch.empty((n_seg, C), dtype=torch.float32, device=u.device)
     slot_stride = state.stride(0) if state.shape[0] > 1 else max(C, state.stride(0))
