@@ -29,13 +29,15 @@ __global__ __launch_bounds__(1024) void post_norm_kernel(float* __restrict__ x, 
     const size_t r = blockIdx.x;
     float* xr = x + r * H;
     const TD* dr = delta ? delta + r * H : nullptr;
-    float v[ITEMS];
+    float v[ITEMS], wv[ITEMS];
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         const int i = it * blockDim.x + threadIdx.x;
         float a = 0.f;
+        wv[it] = 0.f;
         if (i < H) {
+            wv[it] = w[i];                  // (asked for with the row, not behind the block's sum)
             a = alpha * xr[i];
             if (dr) a += pn_sum_parts(dr, (size_t)i, parts, part_stride);
         }
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(1024) void post_norm_kernel(float* __restrict__ x, 
     for (int it = 0; it < ITEMS; ++it) {
         const int i = it * blockDim.x + threadIdx.x;
         if (i < H) {
-            const float o = v[it] * inv * w[i];
+            const float o = v[it] * inv * wv[it];
             xr[i] = o;
             if (rows) store_f32(rows + r * H + i, o);
         }
