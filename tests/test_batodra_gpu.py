@@ -539,3 +539,83 @@ def test_the_command_line_on_a_model_of_the_design(tmp_path):
     p = run("--model", str(out), "--bench", "--batch", "2", "-n", "8", "--prompt-len", "20", "--max-context", "64")
     assert p.returncode == 0, p.stderr[-2000:]
     assert "decode" in (p.stdout + p.stderr)
+
+
+# ---------------------------------------------------------------------------
+# configurations drawn at random
+# ---------------------------------------------------------------------------
+def random_batodra_config(seed: int) -> dict:
+    """Everything config.json can vary, drawn from a seed: widths and vocabularies that are no power of two, three to
+    seven layers of any type in any order, some of them on an earlier layer's tensors, with or without a feed-forward;
+    head sizes in steps of 8, heads and groups, values wider or narrower than keys, whole or partial rotations with
+    or without stretched frequencies, windows from one key to longer than the test, none to eight kept tokens; one
+    to six taps, one to eight blocks."""
+    rng = np.random.default_rng(7000 + seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+
+    def rot(dim):
+        dims = int(pick([dim, dim, max(2, dim // 2), max(2, (dim // 4) * 2), 2]))
+        scaling = None
+        if pick([True, False]):
+            scaling = (float(pick([2.0, 4.0, 8.0, 32.0])), int(pick([16, 64, 512])), float(pick([4.0, 32.0])), float(pick([0.5, 1.0, 2.0])))
+        return (float(pick([50.0, 1e4, 5e5])), dims, scaling)
+
+    def layer():
+        kind = pick(["rglru", "attention", "attention_2"])
+        ff = pick([None, int(pick([24, 56, 96, 136, 256]))])
+        if kind == "rglru":
+            blocks = int(pick([1, 2, 3, 4, 8]))
+            return bc.recurrent(blocks * int(pick([8, 12, 16, 32, 40, 64])), blocks, int(pick([1, 2, 3, 4, 6])), ff=ff)
+        kv = int(pick([1, 2, 3, 4]))
+        heads = kv * int(pick([1, 1, 2, 3, 4]))
+        if kind == "attention":
+            dim = int(pick([8, 16, 24, 32, 32, 64, 64, 128]))
+            dv = int(pick([dim, 2 * dim, 16, 40, 64, 128]))
+            return bc.differential(heads, kv, dim, dv, float(pick([dim ** -0.5, 0.3, 0.1])), float(pick([0.2, 0.5, 0.8])), rot(dim)[:2] +
+                                   ((rot(dim)[2],) if pick([False, False, True]) else ()), ff=ff)
+        dim = int(pick([8, 16, 24, 40, 64, 64, 96, 128]))
+        dv = int(pick([dim, dim, 16, 48, 64, 128]))
+        return bc.windowed(heads, kv, dim, dv, float(pick([8.0, 12.0, 4.0])) / dim, rot(dim), int(pick([1, 5, 33, 40, 64, 65, 100, 1000])),
+                           int(pick([0, 0, 1, 4, 6, 8])), ff=ff)
+
+    layers = []
+    for i in range(int(pick([3, 4, 5, 6, 7]))):
+        if layers and pick([True, False, False]):
+            src = int(rng.integers(0, len(layers)))
+            src = layers[src].get("weights_of", src)
+            new = {k: v for k, v in layers[src].items()}
+            new["weights_of"] = src
+            layers.append(new)
+        else:
+            layers.append(layer())
+    return {"architecture": "Batodra", "vocab": int(pick([67, 131, 256, 577, 1000])), "width": int(pick([40, 64, 72, 96, 136, 192, 256])),
+            "norm": {"eps": float(pick([1e-6, 1e-5, 1e-4]))}, "postln_alpha": float(pick([1.0, 1.5, 2.5, 4.0])), "layers": layers,
+            "torch_dtype": "bfloat16"}
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("seed", list(range(16)))
+def test_random_configuration(seed, dtype):
+    """Ragged prompts in one step, single tokens with a sequence ending early, then a continued prompt beside a new one
+    in the freed slot, against the plain implementation."""
+    name = f"random_{seed}"
+    bc.ALL[name] = random_batodra_config(seed)
+    rng = np.random.default_rng(seed)
+    lens = [int(rng.integers(1, 150)) for _ in range(3)]
+    seqs = [H.tokens(name, n + 8, 10 * seed + i) for i, n in enumerate(lens)]
+    plain = [H.plain_logits(name, s) for s in seqs]
+    eng = H.engine(name, dtype, max_tokens=64 * 12, n_slots=3)
+    slots = [eng.alloc_slot() for _ in seqs]
+    got = eng.step([(sl, list(s[:n])) for sl, s, n in zip(slots, seqs, lens)], want="all")
+    H.close(_np(got), np.concatenate([p[:n] for p, n in zip(plain, lens)]), dtype, f"{name}: prompts")
+    live = [0, 1, 2]
+    for t in range(6):
+        if t == 3:                                      # the second sequence ends early; its slot takes a new prompt later
+            eng.free_slot(slots[1])
+            live = [0, 2]
+        got = eng.step([(slots[i], [seqs[i][lens[i] + t]]) for i in live], want="last")
+        H.close(_np(got), np.stack([plain[i][lens[i] + t] for i in live]), dtype, f"{name}: token {t}")
+    slots[1] = eng.alloc_slot()
+    got = eng.step([(slots[0], list(seqs[0][lens[0] + 6:lens[0] + 8])), (slots[1], list(seqs[1][:lens[1]]))], want=[[0, 1], [lens[1] - 1]])
+    want = np.stack([plain[0][lens[0] + 6], plain[0][lens[0] + 7], plain[1][lens[1] - 1]])
+    H.close(_np(got), want, dtype, f"{name}: a continued prompt beside a new one")
