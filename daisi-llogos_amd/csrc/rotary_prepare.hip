@@ -8,7 +8,7 @@
 //     1: (2i, 2i + 1);
 //   - optionally (unit_after) division by the unit's root mean square, without a weight (after the rotation).
 // A kv head's key row in its page is its `maps` units side by side (k_page_dim >= maps * dim values); a value
-// row has v_dim values in pages of v_page_dim.  All arithmetic in 32-bit; one wave a (token, unit).
+// row has v_dim values in pages of v_page_dim.  All arithmetic in 32-bit; 16, 32 or 64 lanes of a wave a (token, unit).
 #include "common.h"
 
 constexpr int kPrepUnitsPerBlock = 4;
@@ -28,8 +28,16 @@ __device__ __forceinline__ float rp_sum_parts(const TI* p, size_t i, int parts, 
     return v;
 }
 
-// R: values a lane holds of a unit (dim <= 64 R).
-template <typename TI, typename T, int R>
+// L lanes of a wave take a unit (a wave takes 64 / L units side by side: a unit of 64 values is a quarter of a
+// wave's worth of work); R: values a lane holds of a unit (dim <= L R).
+template <int L>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int o = L / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+template <typename TI, typename T, int R, int L>
 __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, size_t part_stride, int row_stride,
                                       const float* __restrict__ bias, T* __restrict__ q_out, int n_q, int n_k, int n_v,
                                       int dim, int v_dim, int maps, int rot, int pairing,
@@ -38,11 +46,12 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
                                       PagedKV cache, int v_page_dim, const int* __restrict__ tok_seq,
                                       const int* __restrict__ tok_pos, int lds_row) {
     extern __shared__ float smem[];
+    constexpr int kPerWave = kWave / L;
     const int t = blockIdx.x;
-    const int unit = blockIdx.y * kPrepUnitsPerBlock + threadIdx.y;
-    const int lane = threadIdx.x;
+    const int sub = threadIdx.x / L, lane = threadIdx.x % L;
+    const int unit = (blockIdx.y * kPrepUnitsPerBlock + threadIdx.y) * kPerWave + sub;
     const bool active = unit < n_q + n_k + n_v;
-    float* buf = smem + threadIdx.y * lds_row;
+    float* buf = smem + (threadIdx.y * kPerWave + sub) * lds_row;
     const bool is_q = unit < n_q;
     const bool is_k = !is_q && unit < n_q + n_k;
     const int width = (is_q || is_k) ? dim : v_dim;
@@ -55,7 +64,7 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
 
     float ss = 0.f;
     if (active) {
-        for (int d = lane; d < width; d += kWave) {
+        for (int d = lane; d < width; d += L) {
             float v = rp_sum_parts(src, (size_t)d, parts, part_stride);
             if (bias) v += bias[col0 + d];
             buf[d] = v;
@@ -63,29 +72,28 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
         }
     }
     __syncthreads();
+    ss = group_sum<L>(ss);                                   // (every lane of the wave takes part, whatever its unit)
     if (active && norm_w) {
-        ss = wave_sum(ss);
         const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
-        for (int d = lane; d < dim; d += kWave) buf[d] = buf[d] * inv * norm_w[d];
+        for (int d = lane; d < dim; d += L) buf[d] = buf[d] * inv * norm_w[d];
     }
     __syncthreads();
-    if (!active) return;
-    if (!is_q && !is_k) {
+    if (active && !is_q && !is_k) {
         const int vh = unit - n_q - n_k;
         T* vdst = v_pool + paged_base(cache, tok_seq[t], vh, pos) / cache.head_dim * v_page_dim;
-        for (int d = lane; d < v_dim; d += kWave) store_f32(vdst + page_value_offset(in_page, d), buf[d]);
-        return;
+        for (int d = lane; d < v_dim; d += L) store_f32(vdst + page_value_offset(in_page, d), buf[d]);
     }
+    const bool turns = active && (is_q || is_k);
     const int half = rot / 2;
     const float2* c = cs + (size_t)t * half;
-    // a lane's rotated values: dimensions lane, lane + 64, ... (both partners are read before either is stored)
+    // a lane's rotated values: dimensions lane, lane + L, ... (both partners are read before either is stored)
     float mine[R];
     float s2 = 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int d = lane + r * kWave;
+        const int d = lane + r * L;
         float v = 0.f;
-        if (d < dim) {
+        if (turns && d < dim) {
             v = buf[d];
             if (d < rot) {
                 if (pairing == 0) {
@@ -102,12 +110,13 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
         s2 += v * v;
     }
     float after = 1.f;
-    if (unit_after) after = 1.0f / sqrtf(wave_sum(s2) / (float)dim + eps);
+    if (unit_after) after = 1.0f / sqrtf(group_sum<L>(s2) / (float)dim + eps);
+    if (!turns) return;
     if (is_q) {
         T* dst = q_out + ((size_t)t * n_q + unit) * dim;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int d = lane + r * kWave;
+            const int d = lane + r * L;
             if (d < dim) store_f32(dst + d, mine[r] * after);
         }
     } else {
@@ -116,7 +125,7 @@ __global__ void rotary_prepare_kernel(const TI* __restrict__ qkv, int parts, siz
         const int col = (ku % maps) * dim;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int d = lane + r * kWave;
+            const int d = lane + r * L;
             if (d < dim) store_f32(dst + page_key_offset(in_page, col + d, cache.head_dim), mine[r] * after);
         }
     }
@@ -139,18 +148,23 @@ LLOGOS_EXPORT int llogos_rotary_prepare(const void* qkv, int in_dtype, int parts
     PagedKV cache{table, table_stride, n_kv, k_page_dim > 0 ? k_page_dim : 1};
     const int units = n_q + n_k + n_v;
     const int lds_row = dim > v_dim ? dim : v_dim;
-    dim3 grid(T, (units + kPrepUnitsPerBlock - 1) / kPrepUnitsPerBlock), block(kWave, kPrepUnitsPerBlock);
-    const size_t smem = (size_t)kPrepUnitsPerBlock * lds_row * sizeof(float);
-#define LAUNCH_R(TI, T_, R_) rotary_prepare_kernel<TI, T_, R_><<<grid, block, smem, stream>>>( \
+    // lanes a unit: 16 up to 64 values, 32 up to 128, else the wave
+    int lanes = dim <= 64 ? 16 : (dim <= 128 ? 32 : kWave);
+    while (lanes < kWave && (size_t)kPrepUnitsPerBlock * (kWave / lanes) * lds_row * sizeof(float) > 32 * 1024) lanes *= 2;   // (wide values beside narrow keys)
+    const int per_block = kPrepUnitsPerBlock * (kWave / lanes);
+    dim3 grid(T, (units + per_block - 1) / per_block), block(kWave, kPrepUnitsPerBlock);
+    const size_t smem = (size_t)per_block * lds_row * sizeof(float);
+    if (smem > 64 * 1024) return LLOGOS_TOO_LARGE;
+#define LAUNCH_RL(TI, T_, R_, L_) rotary_prepare_kernel<TI, T_, R_, L_><<<grid, block, smem, stream>>>( \
         (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_q, n_k, n_v, dim, v_dim, maps, rot, pairing, \
         q_norm_w, k_norm_w, unit_after, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, v_page_dim, tok_seq, tok_pos, lds_row)
-#define LAUNCH(TI, T_) do { if (dim <= kWave) LAUNCH_R(TI, T_, 1); else if (dim <= 2 * kWave) LAUNCH_R(TI, T_, 2); \
-        else if (dim <= 4 * kWave) LAUNCH_R(TI, T_, 4); else LAUNCH_R(TI, T_, kPrepMaxDim / kWave); } while (0)
+#define LAUNCH(TI, T_) do { if (lanes == 16) LAUNCH_RL(TI, T_, 4, 16); else if (lanes == 32) LAUNCH_RL(TI, T_, 4, 32); \
+        else if (dim <= 4 * kWave) LAUNCH_RL(TI, T_, 4, kWave); else LAUNCH_RL(TI, T_, kPrepMaxDim / kWave, kWave); } while (0)
     if (dtype == DT_F32 && in_dtype == DT_F32) LAUNCH(float, float);
     else if (dtype == DT_BF16 && in_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
     else if (dtype == DT_BF16 && in_dtype == DT_F32) LAUNCH(float, bf16_t);
     else return LLOGOS_BAD_ARGUMENT;
 #undef LAUNCH
-#undef LAUNCH_R
+#undef LAUNCH_RL
     return LLOGOS_LAUNCH_CHECK();
 }
