@@ -29,18 +29,38 @@ __global__ __launch_bounds__(1024) void post_norm_kernel(float* __restrict__ x, 
     const size_t r = blockIdx.x;
     float* xr = x + r * H;
     const TD* dr = delta ? delta + r * H : nullptr;
-    float v[ITEMS], wv[ITEMS];
+    float v[ITEMS], wv[ITEMS], xv[ITEMS], sum[ITEMS];
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         const int i = it * blockDim.x + threadIdx.x;
-        float a = 0.f;
-        wv[it] = 0.f;
-        if (i < H) {
-            wv[it] = w[i];                  // (asked for with the row, not behind the block's sum)
-            a = alpha * xr[i];
-            if (dr) a += pn_sum_parts(dr, (size_t)i, parts, part_stride);
+        wv[it] = i < H ? w[i] : 0.f;        // (asked for with the row, not behind the block's sum)
+        xv[it] = i < H ? xr[i] : 0.f;
+        sum[it] = (dr && i < H) ? load_f32(dr + i) : 0.f;
+    }
+    // the product's other parts, four at a time for all of the thread's values at once (their loads are in flight
+    // together), added in ascending order
+    if (dr) {
+        for (int q0 = 1; q0 < parts; q0 += 4) {
+            float y[4][ITEMS];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int it = 0; it < ITEMS; ++it) {
+                    const int i = it * blockDim.x + threadIdx.x;
+                    y[j][it] = (q0 + j < parts && i < H) ? load_f32(dr + (size_t)(q0 + j) * part_stride + i) : 0.f;
+                }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (q0 + j < parts) {
+#pragma unroll
+                    for (int it = 0; it < ITEMS; ++it) sum[it] += y[j][it];
+                }
         }
+    }
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const float a = alpha * xv[it] + sum[it];
         v[it] = a;
         ss += a * a;
     }
