@@ -93,6 +93,7 @@ class Rotary(PositionEncoding):
             elif kind not in (None, "default"):
                 raise ValueError(f"unknown rotary scaling '{kind}'")
         self.freqs = freqs
+        self.table_key = ("rotary", self.amplitude, tuple(freqs))
         self.inv_freq: Optional[torch.Tensor] = None
 
     def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
@@ -101,7 +102,8 @@ class Rotary(PositionEncoding):
 
     def prepare(self, ctx: StepContext) -> torch.Tensor:
         """(cos, sin) table [T, rot/2, 2] of the step's positions, made once per step."""
-        key = ("rotary", id(self))
+        # rotations with the same frequencies and amplitude (several layers of one kind) share the step's table
+        key = self.table_key
         table = ctx.shared.get(key)
         if table is None:
             table = K.rope_table(ctx.tok_pos, self.inv_freq, self.amplitude)
