@@ -82,3 +82,12 @@ def _batodra() -> None:
 
 
 _batodra()
+
+
+def _zasidra() -> None:
+    from ..models.zasidra import zasidra_spec
+    from .zasidra_config import ZasidraConfig
+    register_architecture("Zasidra", ZasidraConfig.from_dict, zasidra_spec)
+
+
+_zasidra()

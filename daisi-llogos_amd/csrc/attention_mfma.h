@@ -291,10 +291,10 @@ __device__ __forceinline__ void softmax_page_bent(f32x4 (&s)[4], WaveState<VP>& 
     }
 }
 
-// What finishes a row: the sink's share of the denominator (exp(0 - max), the maximum being in units of
-// log2) and the head's gate.  Returns the factor on the unnormalised output.
-__device__ __forceinline__ float finish_factor(float m, float l, int unit_sink, const float* gate_logit) {
-    if (unit_sink) l += __builtin_amdgcn_exp2f(-m);
+// What finishes a row: the sink's share of the denominator (exp(sink - max): `sink` points at the head's sink
+// score, the maximum is in units of log2) and the head's gate.  Returns the factor on the unnormalised output.
+__device__ __forceinline__ float finish_factor(float m, float l, const float* sink, const float* gate_logit) {
+    if (sink) l += __builtin_amdgcn_exp2f(*sink * kLog2e - m);
     float f = l > 0.f ? 1.0f / l : 0.f;
     if (gate_logit) f *= 1.0f / (1.0f + expf(-*gate_logit));
     return f;
@@ -325,7 +325,7 @@ struct DirectPageLds {
 // wave a SIMD cannot overlap its matrix and its vector instructions), so a prompt of few tiles
 // took as long as the pages of its last tile, one after the other.
 // VD: the values' width where it is not the keys' (HD); BENT: the scores are scaled and bent through a tanh before
-// the softmax (cap > 0), a row may end with a sink of score 0 in its denominator (unit_sink) and with a gate on its
+// the softmax (cap > 0), a row may end with a sink in its denominator (head_sink: a score a head) and with a gate on its
 // head (gate [tokens, gate_stride] logits), and there is no window.
 // MAPS = 2: every head has two score maps over the same values (differential attention).  A map is a head of its own
 // here: the caller gives twice the heads and twice the group, head 2 h + m is map m of head h; a kv head's key row
@@ -338,7 +338,7 @@ void attn_prefill_direct_kernel(
         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
         const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
         const int* __restrict__ tok_pos, int batch, int n_tiles, int n_heads, int n_kv_heads, int group,
-        float scale, int window, int sinks, float cap = 0.f, int unit_sink = 0, const float* __restrict__ gate = nullptr,
+        float scale, int window, int sinks, float cap = 0.f, const float* __restrict__ head_sink = nullptr, const float* __restrict__ gate = nullptr,
         int gate_stride = 0) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int set = HALVES == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / (kAttnWaves * kWave)) : 0;
@@ -581,7 +581,7 @@ void attn_prefill_direct_kernel(
     }
     auto write_out = [&](const WaveState<VD>& st, int rr) {
         if (rr >= wave_rows) return;
-        const float inv = BENT ? finish_factor(st.m, st.l, unit_sink, gate ? gate + (size_t)(row0 + rr) * gate_stride + h : nullptr)
+        const float inv = BENT ? finish_factor(st.m, st.l, head_sink ? head_sink + h : nullptr, gate ? gate + (size_t)(row0 + rr) * gate_stride + h : nullptr)
                                : (st.l > 0.f ? 1.0f / st.l : 0.f);
         if (MAPS > 1) {
             float* frow = reinterpret_cast<float*>(out) + ((size_t)(row0 + rr) * n_heads + h) * VD;

@@ -1,6 +1,6 @@
 // bfloat16 attention on the matrix cores for heads whose keys and values have different widths,
 // whose scores may be bent through a tanh (s -> cap * tanh(s / cap)), whose softmax may carry a
-// sink of score 0 (one added to the denominator) and whose output may be gated head by head
+// sink (a score a head without a key or a value: exp(sink) joins the denominator) and whose output may be gated head by head
 // (sigmoid of a logit a token and head).  No window: a query sees every key up to its own.
 //
 // Keys are rows of KP = 32 KS dimensions in their pages, values rows of VP = 16 VB; the pages are
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per
         bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
         const bf16_t* __restrict__ v_pool, const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
         const int* __restrict__ tok_pos, int batch, int n_heads, int n_kv_heads, int group, float scale, float cap,
-        int unit_sink, const float* __restrict__ gate, int gate_stride) {
+        const float* __restrict__ head_sink, const float* __restrict__ gate, int gate_stride) {
     constexpr int KP = 32 * KS, VP = 16 * VB;
     int tile = blockIdx.x, b = 0, first = 0;
     for (; b < batch; ++b) {
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per
         weigh_values<VP>(st, vf, pf, corr, min(kPageTokens, written - key0));
     }
     if (!col_ok) return;
-    const float f = finish_factor(st.m, st.l, unit_sink, gate ? gate + (size_t)my_row * gate_stride + h : nullptr);
+    const float f = finish_factor(st.m, st.l, head_sink ? head_sink + h : nullptr, gate ? gate + (size_t)my_row * gate_stride + h : nullptr);
     bf16_t* orow = out + ((size_t)my_row * n_heads + h) * VP;
 #pragma unroll
     for (int db = 0; db < VB; ++db) {
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void capped_decode_kernel(
         bf16_t* __restrict__ out, float* __restrict__ partial, const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
         const int* __restrict__ tok_pos, int n_heads, int n_kv_heads, int group, float scale, float cap, int ppw,
-        int unit_sink, const float* __restrict__ gate, int gate_stride) {
+        const float* __restrict__ head_sink, const float* __restrict__ gate, int gate_stride) {
     constexpr int KP = 32 * KS, VP = 16 * VB, WAVES = kAttnWaves;
     extern __shared__ float lds[];
     float* lds_m = lds;
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void capped_decode_kernel(
         }
         const int head = kvh * group + col;
         if (n_z == 1) {
-            const float f = finish_factor(m, l, unit_sink, gate ? gate + (size_t)b * gate_stride + head : nullptr);
+            const float f = finish_factor(m, l, head_sink ? head_sink + head : nullptr, gate ? gate + (size_t)b * gate_stride + head : nullptr);
             out[((size_t)b * n_heads + head) * VP + d] = f32_to_bf16(o * f);
         } else {
             float* dst = partial + (((size_t)b * n_heads + head) * n_z + z) * (VP + 2);
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void capped_decode_kernel(
 template <int VB>
 __global__ __launch_bounds__(16 * VB) void capped_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial,
                                                                const int* __restrict__ tok_pos, int n_heads, int n_z,
-                                                               int pages_per_block, int unit_sink,
+                                                               int pages_per_block, const float* __restrict__ head_sink,
                                                                const float* __restrict__ gate, int gate_stride) {
     constexpr int VP = 16 * VB;
     const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(16 * VB) void capped_merge_kernel(bf16_t* __restric
         l += p[1] * f;
         o += p[2 + d] * f;
     }
-    const float f = finish_factor(m, l, unit_sink, gate ? gate + (size_t)b * gate_stride + h : nullptr);
+    const float f = finish_factor(m, l, head_sink ? head_sink + h : nullptr, gate ? gate + (size_t)b * gate_stride + h : nullptr);
     out[((size_t)b * n_heads + h) * VP + d] = f32_to_bf16(o * f);
 }
 
@@ -263,7 +263,7 @@ static int capped_pages_per_wave(int batch, int n_kv_heads, int table_width) {
 LLOGOS_EXPORT int llogos_capped_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                                                   const int* table, int table_stride, const int* cu, const int* tok_pos,
                                                   int batch, int n_tiles, int n_heads, int n_kv_heads, int dk, int dv, float scale,
-                                                  float softcap, int unit_sink, const float* gate, int gate_stride,
+                                                  float softcap, const float* head_sink, const float* gate, int gate_stride,
                                                   int tile_rows, int halves, hipStream_t stream) {
     if (batch <= 0 || n_tiles <= 0 || softcap < 0.f || (gate && gate_stride < n_heads)) return LLOGOS_BAD_ARGUMENT;
     if ((tile_rows != 64 && tile_rows != kTileRows) || (halves != 1 && halves != 2)) return LLOGOS_BAD_ARGUMENT;
@@ -282,7 +282,7 @@ LLOGOS_EXPORT int llogos_capped_attn_prefill_bf16(void* out, const void* q, int 
         if (e != hipSuccess) return (int)e; \
         attn_prefill_direct_kernel<32 * KS, HALVES, 16 * VB, true><<<lgrid, HALVES * kAttnWaves * kWave, smem, stream>>>( \
             (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
-            cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, 0, 0, softcap, unit_sink, gate, gate_stride); \
+            cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, 0, 0, softcap, head_sink, gate, gate_stride); \
         return LLOGOS_LAUNCH_CHECK(); } while (0)
 #define DIRECT1(KS, VB) DIRECT(KS, VB, 1)
 #define DIRECT2(KS, VB) DIRECT(KS, VB, 2)
@@ -293,7 +293,7 @@ LLOGOS_EXPORT int llogos_capped_attn_prefill_bf16(void* out, const void* q, int 
     }
 #define PRE(KS, VB) capped_prefill_kernel<KS, VB><<<grid, kAttnWaves * kWave, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, q_stride, \
         (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, cu, tok_pos, batch, n_heads, n_kv_heads, group, scale, \
-        softcap, unit_sink, gate, gate_stride)
+        softcap, head_sink, gate, gate_stride)
     CAPPED_SHAPES(PRE)
 #undef PRE
     return LLOGOS_LAUNCH_CHECK();
@@ -309,7 +309,7 @@ LLOGOS_EXPORT long long llogos_capped_attn_decode_workspace(int batch, int n_hea
 LLOGOS_EXPORT int llogos_capped_attn_decode_bf16(void* out, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                                                  const int* table, int table_stride, int table_width, const int* tok_pos,
                                                  int batch, int n_heads, int n_kv_heads, int dk, int dv, float scale,
-                                                 float softcap, int unit_sink, const float* gate, int gate_stride,
+                                                 float softcap, const float* head_sink, const float* gate, int gate_stride,
                                                  float* workspace, long long workspace_floats, hipStream_t stream) {
     if (batch <= 0 || table_width <= 0 || softcap < 0.f || (gate && gate_stride < n_heads)) return LLOGOS_BAD_ARGUMENT;
     if (!capped_shape_ok(n_heads, n_kv_heads, dk, dv) || q_stride % 8) return LLOGOS_UNSUPPORTED;
@@ -321,13 +321,13 @@ LLOGOS_EXPORT int llogos_capped_attn_decode_bf16(void* out, const void* q, int q
     const size_t lds = (size_t)kAttnWaves * (group * (dv + 1) + 32) * sizeof(float);
 #define DEC(KS, VB) capped_decode_kernel<KS, VB><<<grid, kAttnWaves * kWave, lds, stream>>>((bf16_t*)out, workspace, (const bf16_t*)q, \
         q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, tok_pos, n_heads, n_kv_heads, group, scale, \
-        softcap, ppw, unit_sink, gate, gate_stride)
+        softcap, ppw, head_sink, gate, gate_stride)
     CAPPED_SHAPES(DEC)
 #undef DEC
     if (n_z > 1) {
         dim3 mgrid(batch, n_heads);
 #define MRG(VB) capped_merge_kernel<VB><<<mgrid, 16 * VB, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, n_z, kAttnWaves * ppw, \
-        unit_sink, gate, gate_stride)
+        head_sink, gate, gate_stride)
         if (dv == 64) MRG(4); else if (dv == 80) MRG(5); else if (dv == 96) MRG(6); else MRG(8);
 #undef MRG
     }

@@ -93,10 +93,12 @@ LLOGOS_EXPORT int llogos_latent_prepare(const float* kv, int ldkv, const float* 
 // a: row stride lda, head stride a_head; out: row stride ldo, head stride o_head; w [H, N, K] dense.
 // Tiles of 64 tokens x 64 outputs, 16 values of k at a time through LDS, 4 x 4 outputs a thread,
 // sums in 32-bit in ascending k: an output's sum does not depend on what else is in the step.
+// gate (or null): float32 logits, gate[t * gate_stride + h]; head h's outputs of row t are multiplied by its sigmoid.
 template <typename TA, typename TW, typename TO>
 __global__ __launch_bounds__(256) void head_products_kernel(TO* __restrict__ out, int ldo, int o_head,
                                                             const TA* __restrict__ a, int lda, int a_head,
-                                                            const TW* __restrict__ w, int M, int N, int K) {
+                                                            const TW* __restrict__ w, int M, int N, int K,
+                                                            const float* __restrict__ gate, int gate_stride) {
     __shared__ float sa[16][64 + 4];
     __shared__ float sw[16][64 + 4];
     const int h = blockIdx.z, m0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
@@ -127,10 +129,11 @@ __global__ __launch_bounds__(256) void head_products_kernel(TO* __restrict__ out
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + ty * 4 + i;
         if (m >= M) continue;
+        const float f = gate ? 1.0f / (1.0f + expf(-gate[(size_t)m * gate_stride + h])) : 1.0f;
 #pragma unroll
         for (int jn = 0; jn < 4; ++jn) {
             const int n = n0 + tx * 4 + jn;
-            if (n < N) store_f32(out + (size_t)m * ldo + (size_t)h * o_head + n, acc[i][jn]);
+            if (n < N) store_f32(out + (size_t)m * ldo + (size_t)h * o_head + n, gate ? acc[i][jn] * f : acc[i][jn]);
         }
     }
 }
@@ -142,7 +145,8 @@ __global__ __launch_bounds__(256) void head_products_kernel(TO* __restrict__ out
 // rounded up to 1, 2, 4, 8 or 16 (rows that are not there are zeros in LDS).
 template <int TMAX, int KG, typename TA, typename TW, typename TO>
 __global__ __launch_bounds__(64 * KG) void head_products_few_kernel(TO* __restrict__ out, int ldo, int o_head, const TA* __restrict__ a, int lda, int a_head,
-                                         const TW* __restrict__ w_kn, int M, int N, int K) {
+                                         const TW* __restrict__ w_kn, int M, int N, int K,
+                                         const float* __restrict__ gate, int gate_stride) {
     // LDS: the head's rows as [k][TMAX] (one or two 16-byte reads bring every row's value of a k), then the KG
     // k-groups' sums [KG][64][TMAX]
     extern __shared__ float rows_lds[];
@@ -183,6 +187,7 @@ __global__ __launch_bounds__(64 * KG) void head_products_few_kernel(TO* __restri
             float v = sums[nl * TMAX + t];
 #pragma unroll
             for (int j = 1; j < KG; ++j) v += sums[(j * 64 + nl) * TMAX + t];          // in the groups' order
+            if (t < M && gate) v *= 1.0f / (1.0f + expf(-gate[(size_t)t * gate_stride + h]));
             if (t < M) store_f32(out + (size_t)t * ldo + (size_t)h * o_head + n, v);
         }
     }
@@ -190,8 +195,8 @@ __global__ __launch_bounds__(64 * KG) void head_products_few_kernel(TO* __restri
 
 LLOGOS_EXPORT int llogos_head_products_few(void* out, int out_dtype, int ldo, int o_head, const void* a, int a_dtype, int lda,
                                            int a_head, const void* w_kn, int w_dtype, int M, int H, int N, int K,
-                                           hipStream_t stream) {
-    if (M <= 0 || M > 16 || H <= 0 || N <= 0 || K <= 0) return LLOGOS_BAD_ARGUMENT;
+                                           const float* gate, int gate_stride, hipStream_t stream) {
+    if (M <= 0 || M > 16 || H <= 0 || N <= 0 || K <= 0 || (gate && gate_stride < H)) return LLOGOS_BAD_ARGUMENT;
     int tmax = 1;
     while (tmax < M) tmax <<= 1;
     // sixteen groups of k where their sums fit beside the rows and every group has k of its own, else four
@@ -205,13 +210,13 @@ LLOGOS_EXPORT int llogos_head_products_few(void* out, int out_dtype, int ldo, in
                 hipError_t e = hipFuncSetAttribute((const void*)head_products_few_kernel<TM, 16, TA, TW, TO>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
                 if (e != hipSuccess) return (int)e; \
             } \
-            head_products_few_kernel<TM, 16, TA, TW, TO><<<grid, 1024, smem, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K); \
+            head_products_few_kernel<TM, 16, TA, TW, TO><<<grid, 1024, smem, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K, gate, gate_stride); \
         } else { \
             if (smem > 48 * 1024) { \
                 hipError_t e = hipFuncSetAttribute((const void*)head_products_few_kernel<TM, 4, TA, TW, TO>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
                 if (e != hipSuccess) return (int)e; \
             } \
-            head_products_few_kernel<TM, 4, TA, TW, TO><<<grid, 256, smem, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K); \
+            head_products_few_kernel<TM, 4, TA, TW, TO><<<grid, 256, smem, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K, gate, gate_stride); \
         } } while (0)
 #define HPT(TA, TW, TO) do { if (tmax == 1) HPF(1, TA, TW, TO); else if (tmax == 2) HPF(2, TA, TW, TO); else if (tmax == 4) HPF(4, TA, TW, TO); \
                              else if (tmax == 8) HPF(8, TA, TW, TO); else HPF(16, TA, TW, TO); } while (0)
@@ -227,11 +232,12 @@ LLOGOS_EXPORT int llogos_head_products_few(void* out, int out_dtype, int ldo, in
 }
 
 LLOGOS_EXPORT int llogos_head_products(void* out, int out_dtype, int ldo, int o_head, const void* a, int a_dtype, int lda,
-                                       int a_head, const void* w, int w_dtype, int M, int H, int N, int K, hipStream_t stream) {
-    if (M <= 0 || H <= 0 || N <= 0 || K <= 0) return LLOGOS_BAD_ARGUMENT;
+                                       int a_head, const void* w, int w_dtype, int M, int H, int N, int K,
+                                       const float* gate, int gate_stride, hipStream_t stream) {
+    if (M <= 0 || H <= 0 || N <= 0 || K <= 0 || (gate && gate_stride < H)) return LLOGOS_BAD_ARGUMENT;
     dim3 grid((M + 63) / 64, (N + 63) / 64, H);
 #define HP(TA, TW, TO) head_products_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, \
-        (const TW*)w, M, N, K)
+        (const TW*)w, M, N, K, gate, gate_stride)
     if (a_dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32) HP(float, float, float);
     else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_F32) HP(float, bf16_t, float);
     else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HP(float, bf16_t, bf16_t);

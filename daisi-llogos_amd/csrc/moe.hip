@@ -1,6 +1,8 @@
-// A mixture of experts whose choice is a table over token ids: token t goes to the `top` experts
-// table[ids[t]][0..top), each weighted alike.  Everything is decided on the device from the step's
-// ids, so a captured step replays with other tokens.
+// Mixtures of experts.  The choice is either a table over token ids (token t goes to the `top` experts
+// table[ids[t]][0..top), each weighted alike) or a router's (moe_router_logits, moe_router_choose: a
+// softmax over the router's outputs, a correction added for the choice alone, the best groups of
+// neighbouring experts, the `top` best of those, weights from the uncorrected scores).  Everything is
+// decided on the device, so a captured step replays with other tokens.
 //
 //   moe_route    (token, choice) pairs sorted by expert: order[], the experts' segments seg[], and
 //                where[pair] = the pair's place in that order
@@ -8,6 +10,8 @@
 //                (plain 32-bit FMAs, any storage type), optionally gathering its input rows by pair
 //                and squaring relu in its epilogue
 //   moe_combine  out[t] = mean over choices of the pair rows + sigmoid(gate[t]) * shared[t]
+//   moe_combine_weighted  out[t] = sum over choices of weight * pair row (or weight * the token's own row for a
+//                router output that stands for no expert matrix) + shared[t]
 //
 // A row's sums are taken in the order of k alone, in the blocks of gemm_generic.hip (16 products, 16 of
 // those, then the total), so a token's result does not depend on where it falls in a segment or on
@@ -16,7 +20,7 @@
 
 constexpr int kMoeMaxExperts = 1024;
 
-// One block.  seg has E + 1 entries.
+// One block.  seg has E + 1 entries.  ids null: row t of the table is token t's own (a router's choice [T, top]).
 __global__ __launch_bounds__(1024) void moe_route_kernel(const int* __restrict__ ids, const int* __restrict__ table, int T, int top,
                                                          int E, int* __restrict__ order, int* __restrict__ seg,
                                                          int* __restrict__ where) {
@@ -26,7 +30,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int* __restrict__
     for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
     __syncthreads();
     for (int p = threadIdx.x; p < P; p += blockDim.x) {
-        int e = table[(size_t)ids[p / top] * top + p % top];
+        int e = table[(size_t)(ids ? ids[p / top] : p / top) * top + p % top];
         e = min(max(e, 0), E - 1);
         atomicAdd(&count[e], 1);
     }
@@ -41,7 +45,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int* __restrict__
     for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
     __syncthreads();
     for (int p = threadIdx.x; p < P; p += blockDim.x) {
-        int e = table[(size_t)ids[p / top] * top + p % top];
+        int e = table[(size_t)(ids ? ids[p / top] : p / top) * top + p % top];
         e = min(max(e, 0), E - 1);
         const int at = start[e] + atomicAdd(&count[e], 1);
         order[at] = p;
@@ -56,7 +60,11 @@ LLOGOS_EXPORT int llogos_moe_route(const int* ids, const int* table, int T, int 
     return LLOGOS_LAUNCH_CHECK();
 }
 
+__device__ __forceinline__ float moe_gated(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
+
 // out[r, :] = act(a_row(r) . w[e]^T) * scale for the sorted rows r of expert e's segment.
+// act 0: none; 1: the square of relu; 2: the matrix's rows are gate and up rows in turn (gate 0, up 0, gate 1, ...)
+// and the result has N / 2 columns silu(gate_i) * up_i.
 // a_row(r) = a[order[r] / top] when gather (the step's token rows), else a[r] (rows already sorted).
 // w is [E][N][K].  Tiles of 64 rows x 64 columns; blockIdx.y counts row tiles over all segments.
 constexpr int GM = 64, GN = 64, GK = 16;
@@ -128,6 +136,16 @@ __global__ __launch_bounds__(256) void moe_product_kernel(TO* __restrict__ out, 
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + ty * 4 + i;
         if (m >= m_end) continue;
+        if (act == 2) {                                     // columns in pairs (gate, up): silu(gate) * up
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                const int n = n0 + tx * 4 + j;
+                if (n + 1 >= N) continue;
+                const float gt = acc[i][j] + mid[i][j], up = acc[i][j + 1] + mid[i][j + 1];
+                store_f32(out + (size_t)m * (N / 2) + n / 2, moe_gated(gt, up) * scale);
+            }
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
@@ -143,7 +161,7 @@ __global__ __launch_bounds__(256) void moe_product_kernel(TO* __restrict__ out, 
 LLOGOS_EXPORT int llogos_moe_product(void* out, int out_dtype, const void* a, int a_dtype, const void* w, int w_dtype,
                                      const int* order, const int* seg, int E, int top, int gather, int P, int N, int K,
                                      int lda, int act, float scale, hipStream_t stream) {
-    if (P <= 0 || N <= 0 || K <= 0 || E <= 0 || top <= 0 || lda < K || act < 0 || act > 1) return LLOGOS_BAD_ARGUMENT;
+    if (P <= 0 || N <= 0 || K <= 0 || E <= 0 || top <= 0 || lda < K || act < 0 || act > 2 || (act == 2 && (N & 1))) return LLOGOS_BAD_ARGUMENT;
     if (a_dtype != w_dtype && !(a_dtype == DT_F32)) return LLOGOS_BAD_ARGUMENT;
     const int row_tiles = (P + GM - 1) / GM + E;
     dim3 grid((N + GN - 1) / GN, row_tiles);
@@ -196,6 +214,163 @@ LLOGOS_EXPORT int llogos_moe_combine(float* out, const float* y, const int* wher
     return LLOGOS_LAUNCH_CHECK();
 }
 
+// ---------------------------------------------------------------- a router
+// z[t, e] = w[e, :] . a[t, :] in 32-bit for steps of few rows: a wave a (token, output), lanes along k, the lanes'
+// sums added by the wave's reduction.  w float32 [E, K]; a [T, lda] of any storage type.
+template <typename TA>
+__global__ __launch_bounds__(256) void moe_router_logits_kernel(float* __restrict__ z, const TA* __restrict__ a, int lda,
+                                                                const float* __restrict__ w, int E, int K) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int e = blockIdx.x * 4 + wave, t = blockIdx.y;
+    if (e >= E) return;
+    const TA* ar = a + (size_t)t * lda;
+    const float* wr = w + (size_t)e * K;
+    float acc = 0.f;
+    for (int k = lane; k < K; k += kWave) acc = fmaf(load_f32(ar + k), wr[k], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) z[(size_t)t * E + e] = acc;
+}
+
+LLOGOS_EXPORT int llogos_moe_router_logits(float* z, const void* a, int a_dtype, int lda, const float* w, int T, int E, int K,
+                                           hipStream_t stream) {
+    if (T <= 0 || E <= 0 || K <= 0 || lda < K) return LLOGOS_BAD_ARGUMENT;
+    dim3 grid((E + 3) / 4, T);
+    if (a_dtype == DT_F32) moe_router_logits_kernel<float><<<grid, 256, 0, stream>>>(z, (const float*)a, lda, w, E, K);
+    else if (a_dtype == DT_BF16) moe_router_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>(z, (const bf16_t*)a, lda, w, E, K);
+    else return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// the wave's largest (value, lowest index among equals); every lane returns it
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, kWave);
+        const int oi = __shfl_xor(i, o, kWave);
+        if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+}
+
+// the largest of v[0..n) among the entries with open[.] != 0 (the lowest index among equals; n when none is open)
+__device__ __forceinline__ int wave_best_open(const float* v, const unsigned char* open, int n, int lane) {
+    float bv = -INFINITY;
+    int bi = n;
+    for (int e = lane; e < n; e += kWave)
+        if (open[e] && (bi == n || v[e] > bv)) { bv = v[e]; bi = e; }
+    wave_argmax(bv, bi);
+    return bi;
+}
+
+// One wave a token.  From the router's logits z [T, E] (float32):
+//   s = softmax(z) over all E outputs;  c = s + correction  (the choice's scores; correction may be null)
+//   the E outputs form n_groups equal groups of neighbours; a group's score is its largest c; outputs outside the
+//   `keep` best groups cannot be chosen (n_groups <= 1 or keep >= n_groups: all can)
+//   choice[t, j] = the j-th largest c that can be chosen (the lowest index among equals), j < top
+//   weight[t, j] = s[choice] / (sum_j s[choice_j] + 1e-20) * scale
+// The caller sees to it that the kept groups hold at least `top` outputs.
+__global__ __launch_bounds__(kWave) void moe_router_choose_kernel(const float* __restrict__ z, const float* __restrict__ correction,
+                                                                  int E, int n_groups, int keep, int top, float scale,
+                                                                  int* __restrict__ choice, float* __restrict__ weight) {
+    __shared__ float s[kMoeMaxExperts], c[kMoeMaxExperts], gbest[kMoeMaxExperts], picked_s[kMoeMaxExperts];
+    __shared__ int picked[kMoeMaxExperts];
+    __shared__ unsigned char open[kMoeMaxExperts], gopen[kMoeMaxExperts];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* zr = z + (size_t)t * E;
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += kWave) { const float v = zr[e]; s[e] = v; m = fmaxf(m, v); }
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += kWave) { const float v = expf(s[e] - m); s[e] = v; sum += v; }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += kWave) {
+        const float v = s[e] / sum;
+        s[e] = v;
+        c[e] = correction ? v + correction[e] : v;
+        open[e] = 1;
+    }
+    __syncthreads();
+    if (n_groups > 1 && keep < n_groups) {
+        const int size = E / n_groups;
+        for (int g = lane; g < n_groups; g += kWave) {
+            float b = c[g * size];
+            for (int j = 1; j < size; ++j) b = fmaxf(b, c[g * size + j]);
+            gbest[g] = b;
+            gopen[g] = 1;
+        }
+        __syncthreads();
+        for (int r = 0; r < keep; ++r) {                     // the best group that is still open is kept and closed
+            const int g = wave_best_open(gbest, gopen, n_groups, lane);
+            __syncthreads();
+            if (lane == 0 && g < n_groups) gopen[g] = 0;
+            __syncthreads();
+        }
+        for (int e = lane; e < E; e += kWave) open[e] = gopen[e / size] ? 0 : 1;     // (what is still open was not kept)
+        __syncthreads();
+    }
+    float total = 0.f;
+    for (int j = 0; j < top; ++j) {
+        const int e = min(wave_best_open(c, open, E, lane), E - 1);
+        __syncthreads();
+        if (lane == 0) { open[e] = 0; picked[j] = e; picked_s[j] = s[e]; }
+        __syncthreads();
+        total += s[e];
+    }
+    const float f = scale / (total + 1e-20f);
+    for (int j = lane; j < top; j += kWave) {
+        choice[(size_t)t * top + j] = picked[j];
+        weight[(size_t)t * top + j] = picked_s[j] * f;
+    }
+}
+
+LLOGOS_EXPORT int llogos_moe_router_choose(const float* z, const float* correction, int T, int E, int n_groups, int keep, int top,
+                                           float scale, int* choice, float* weight, hipStream_t stream) {
+    if (T <= 0 || E <= 0 || E > kMoeMaxExperts || top <= 0 || top > E) return LLOGOS_BAD_ARGUMENT;
+    if (n_groups > 1 && (E % n_groups || keep < 1 || (long long)min(keep, n_groups) * (E / n_groups) < top)) return LLOGOS_BAD_ARGUMENT;
+    moe_router_choose_kernel<<<T, kWave, 0, stream>>>(z, correction, E, n_groups, keep, top, scale, choice, weight);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// out[t, :] = sum_j weight[t, j] * row_j + (sum of the parts of shared[t, :]), with row_j = y[where[t * top + j], :] when
+// choice[t, j] < n_real and the token's own row a[t, :] otherwise (a router output without matrices returns its input).
+// y float32 [P, W]; a [T, lda] of any storage type; shared float32 [(parts,) T, W] or null.
+template <typename TA>
+__global__ void moe_combine_weighted_kernel(float* __restrict__ out, const float* __restrict__ y, const int* __restrict__ where,
+                                            const int* __restrict__ choice, const float* __restrict__ weight, int top, int n_real,
+                                            const TA* __restrict__ a, int lda, const float* __restrict__ shared_rows, int parts,
+                                            size_t part_stride, int T, int W) {
+    const int t = blockIdx.x;
+    for (int col = blockIdx.y * blockDim.x + threadIdx.x; col < W; col += gridDim.y * blockDim.x) {
+        float v = 0.f;
+        for (int j = 0; j < top; ++j) {
+            const int p = t * top + j;
+            const float row = choice[p] < n_real ? y[(size_t)where[p] * W + col] : load_f32(a + (size_t)t * lda + col);
+            v = fmaf(weight[p], row, v);
+        }
+        if (shared_rows) {
+            float sh = shared_rows[(size_t)t * W + col];
+            for (int q = 1; q < parts; ++q) sh += shared_rows[q * part_stride + (size_t)t * W + col];
+            v += sh;
+        }
+        out[(size_t)t * W + col] = v;
+    }
+}
+
+LLOGOS_EXPORT int llogos_moe_combine_weighted(float* out, const float* y, const int* where, const int* choice, const float* weight,
+                                              int top, int n_real, const void* a, int a_dtype, int lda, const float* shared_rows,
+                                              int parts, long long part_stride, int T, int W, hipStream_t stream) {
+    if (T <= 0 || W <= 0 || top <= 0 || parts < 1 || lda < W || n_real < 0) return LLOGOS_BAD_ARGUMENT;
+    const int threads = 256;
+    dim3 grid(T, (W + threads - 1) / threads);
+    if (a_dtype == DT_F32)
+        moe_combine_weighted_kernel<float><<<grid, threads, 0, stream>>>(out, y, where, choice, weight, top, n_real, (const float*)a, lda,
+                                                                         shared_rows, parts, (size_t)part_stride, T, W);
+    else if (a_dtype == DT_BF16)
+        moe_combine_weighted_kernel<bf16_t><<<grid, threads, 0, stream>>>(out, y, where, choice, weight, top, n_real, (const bf16_t*)a, lda,
+                                                                          shared_rows, parts, (size_t)part_stride, T, W);
+    else return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
 // ---------------------------------------------------------------- bfloat16 on the matrix cores
 // The same product with v_mfma_f32_16x16x32_bf16: the first operand holds 16 rows of the expert's matrix, the
 // second 16 sorted rows of activations, so that a lane ends with four neighbouring outputs of one row:
@@ -223,6 +398,11 @@ __device__ __forceinline__ void moe_store4(bf16_t* p, float a, float b, float c,
     u.x = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
     u.y = (uint32_t)f32_to_bf16(c) | ((uint32_t)f32_to_bf16(d) << 16);
     *reinterpret_cast<uint2*>(p) = u;
+}
+
+__device__ __forceinline__ void moe_store2(float* p, float a, float b) { *reinterpret_cast<float2*>(p) = make_float2(a, b); }
+__device__ __forceinline__ void moe_store2(bf16_t* p, float a, float b) {
+    *reinterpret_cast<uint32_t*>(p) = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
 }
 
 // which tile of `rows` sorted rows is this block's: expert, first row, end of the expert's segment (expert -1: none)
@@ -273,10 +453,13 @@ __global__ __launch_bounds__(256) void moe_few_kernel(TO* __restrict__ out, cons
     for (int r = 0; r < 4; ++r) {
         v[r] = ((acc[r] + red[0][lane][r]) + red[1][lane][r]) + red[2][lane][r];
         if (act == 1) { v[r] = fmaxf(v[r], 0.f); v[r] *= v[r]; }
-        v[r] *= scale;
+        if (act != 2) v[r] *= scale;
     }
     const int n = n0 + 4 * g;
-    if (m < m_end && n < N) moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
+    if (m < m_end && n < N) {
+        if (act == 2) moe_store2(out + (size_t)m * (N / 2) + n / 2, moe_gated(v[0], v[1]) * scale, moe_gated(v[2], v[3]) * scale);
+        else moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
+    }
 }
 
 constexpr int kMoeBK = 64;      // LDS rows of 64 values of k: 128 bytes, eight pieces of 16
@@ -387,9 +570,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 for (int r = 0; r < 4; ++r) {
                     v[r] = acc[nt][mt][4 * q + r];
                     if (act == 1) { v[r] = fmaxf(v[r], 0.f); v[r] *= v[r]; }
-                    v[r] *= scale;
+                    if (act != 2) v[r] *= scale;
                 }
-                moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
+                if (act == 2) moe_store2(out + (size_t)m * (N / 2) + n / 2, moe_gated(v[0], v[1]) * scale, moe_gated(v[2], v[3]) * scale);
+                else moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
             }
     }
 }
@@ -398,7 +582,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 LLOGOS_EXPORT int llogos_moe_product_bf16(void* out, int out_dtype, const void* a, const void* w, const int* order, const int* seg,
                                           int E, int top, int gather, int P, int N, int K, int lda, int act, float scale, int form,
                                           hipStream_t stream) {
-    if (P <= 0 || N <= 0 || K <= 0 || E <= 0 || top <= 0 || lda < K || act < 0 || act > 1 || form < 0 || form > 2) return LLOGOS_BAD_ARGUMENT;
+    if (P <= 0 || N <= 0 || K <= 0 || E <= 0 || top <= 0 || lda < K || act < 0 || act > 2 || form < 0 || form > 2) return LLOGOS_BAD_ARGUMENT;
     if ((K % 8) || (N % 4) || (lda % 8) || ((uintptr_t)a % 16) || ((uintptr_t)w % 16) || ((uintptr_t)out % 16)) return LLOGOS_UNSUPPORTED;
     if (out_dtype != DT_F32 && out_dtype != DT_BF16) return LLOGOS_BAD_ARGUMENT;
     const int rows = form == 0 ? 16 : (form == 1 ? 64 : 128);

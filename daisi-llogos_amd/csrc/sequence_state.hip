@@ -598,9 +598,17 @@ __global__ __launch_bounds__(1024) void sandwich_norm_kernel(float* __restrict__
         v[it] = t;
         ss = fmaf(t, t, ss);
     }
-    if (!wn) return;
-    const float inv_x = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
+    if (!h) return;
     TH* hr = h + r * H;
+    if (!wn) {                       // the completed rows as they are, in the reader's type
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+            const int i = it * blockDim.x + threadIdx.x;
+            if (i < H) store_f32(hr + i, v[it]);
+        }
+        return;
+    }
+    const float inv_x = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         const int i = it * blockDim.x + threadIdx.x;

@@ -346,19 +346,26 @@ def _page_dims(k_pool: torch.Tensor, v_pool: Optional[torch.Tensor], n_kv_heads:
 def qkv_prepare(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype, n_heads: int, n_kv_heads: int,
                 head_dim: int, v_dim: int, q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
                 temp_coef: float, temp_every: int, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
-                table: Optional[torch.Tensor], writes: bool = True) -> torch.Tensor:
+                table: Optional[torch.Tensor], writes: bool = True, cs: Optional[torch.Tensor] = None, rot: int = 0,
+                pairing: int = 0) -> torch.Tensor:
     """From projected rows [q | k | v | ...] (float32 [T, >= W] or partial sums [parts, T, >= W], plus `bias`
     [W], W = n_heads * head_dim + n_kv_heads * (head_dim + v_dim)): an RMS norm over the whole of q and of
-    k where a weight is given ([n_heads * head_dim], [n_kv_heads * head_dim]), the query's factor
-    1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1); q comes back [T, n_heads * head_dim] in
-    `out_dtype`, k and v go to their pages.  writes False: only q is made."""
+    k where a weight is given ([n_heads * head_dim], [n_kv_heads * head_dim]), then the rotation of the first
+    `rot` dimensions of every head of q and k by the table `cs` [T, rot / 2, 2] (pairing 0: dimension i with
+    i + rot / 2, 1: 2i with 2i + 1), the query's factor 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1);
+    q comes back [T, n_heads * head_dim] in `out_dtype`, k and v go to their pages.  writes False: only q is
+    made (the rows then need hold no more than q)."""
     _need(qkv.is_cuda and qkv.dtype == torch.float32 and qkv.stride(-1) == 1, "qkv_prepare: float32 rows on the GPU")
     _dev(bias, q_norm_w, k_norm_w, table, ctx.tok_seq, ctx.tok_pos)
     parts, part_stride = _parts(qkv)
     T = qkv.shape[-2]
     Wq, Wk, Wv = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_dim
-    width = Wq + Wk + Wv
+    width = Wq + ((Wk + Wv) if writes else 0)
     _need(qkv.shape[-1] >= width and T == ctx.n_tokens, f"qkv_prepare: rows of at least {width} values, one a token")
+    _need(rot % 2 == 0 and 0 <= rot <= head_dim and pairing in (0, 1), "qkv_prepare: the rotated width must be even and within a head")
+    if rot:
+        _dev(cs)
+        _need(cs is not None and cs.dtype == torch.float32 and tuple(cs.shape) == (T, rot // 2, 2), "qkv_prepare: rotary table shape")
     row_stride = qkv.stride(-2) if T > 1 else max(width, qkv.stride(-2))
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() >= width, f"qkv_prepare: bias must be float32 [{width}]")
@@ -378,7 +385,7 @@ def qkv_prepare(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype:
     _check(_lib().llogos_qkv_prepare(
         _p(qkv), parts, ctypes.c_longlong(part_stride), row_stride, _p(bias), _p(q_out), _DT[out_dtype], n_heads,
         n_kv_heads if writes else 0, head_dim, v_dim, kd, vd, _p(q_norm_w), _p(k_norm_w), ctypes.c_float(eps),
-        ctypes.c_float(temp_coef), int(temp_every), _p(k_pool) if writes else None, _p(v_pool) if writes else None,
+        ctypes.c_float(temp_coef), int(temp_every), _p(cs) if rot else None, int(rot), int(pairing), _p(k_pool) if writes else None, _p(v_pool) if writes else None,
         _p(table) if writes else None, table.stride(0) if (writes and table is not None) else 0, _p(ctx.tok_seq), _p(ctx.tok_pos),
         T, _stream()), "qkv_prepare")
     return q_out
@@ -558,9 +565,10 @@ def scan_plan(batch: int, n_heads: int, dim: int, longest: Optional[int], n_cus:
 
 
 def sandwich_norm(x: torch.Tensor, a: torch.Tensor, post_w: torch.Tensor, next_w: Optional[torch.Tensor], eps: float,
-                  out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+                  out_dtype: torch.dtype, plain_rows: bool = False) -> Optional[torch.Tensor]:
     """x += rmsnorm(a) * post_w in place (x the float32 stream [T, H]; a [T, H] or float32 partial sums
-    [parts, T, H]), and, with next_w, the rows rmsnorm(x) * next_w of the completed stream in `out_dtype`."""
+    [parts, T, H]), and, with next_w, the rows rmsnorm(x) * next_w of the completed stream in `out_dtype`;
+    with plain_rows (and no next_w) the completed rows themselves in `out_dtype`."""
     _dev(x, a, post_w, next_w)
     _need(x.dtype == torch.float32 and x.dim() == 2, "sandwich_norm: x must be float32 [T, H]")
     T, H = x.shape
@@ -568,8 +576,9 @@ def sandwich_norm(x: torch.Tensor, a: torch.Tensor, post_w: torch.Tensor, next_w
     _need(tuple(a.shape[-2:]) == (T, H) and (parts == 1 or a.dtype == torch.float32), "sandwich_norm: a must have x's shape")
     _need(post_w.dtype == torch.float32 and post_w.shape == (H,), "sandwich_norm: weights must be float32 [H]")
     _need(next_w is None or (next_w.dtype == torch.float32 and next_w.shape == (H,)), "sandwich_norm: weights must be float32 [H]")
+    _need(not (plain_rows and next_w is not None), "sandwich_norm: plain rows or the next norm's rows, not both")
     _need(H * 4 <= 65536, "sandwich_norm: rows of more than 16,384 values")
-    h = torch.empty((T, H), dtype=out_dtype, device=x.device) if next_w is not None else None
+    h = torch.empty((T, H), dtype=out_dtype, device=x.device) if (next_w is not None or plain_rows) else None
     if T:
         _check(_lib().llogos_sandwich_norm(_p(x), _p(a), _dt(a), parts, ctypes.c_longlong(part_stride), _p(post_w), _p(next_w),
                                            _p(h), _DT[out_dtype], ctypes.c_float(eps), T, H, _stream()), "sandwich_norm")
@@ -606,34 +615,99 @@ MOE_FEW_PAIRS = 256          # up to so many (token, choice) pairs a step the ex
 MOE_PRODUCT = "auto"         # "auto": chosen by the step; "plain", "few", "tiles64", "tiles128" force a form (tests)
 
 
-def moe_route(ids: torch.Tensor, table: torch.Tensor, n_experts: int):
+def moe_route(ids: Optional[torch.Tensor], table: torch.Tensor, n_experts: int):
     """(order, seg, where) int32 on the device: the step's (token, choice) pairs t * top + j sorted by
     their expert table[ids[t], j], the experts' segments in that order (n_experts + 1 offsets) and each
-    pair's place in it."""
+    pair's place in it.  ids None: table [T, top] holds each token's own choices (a router's)."""
     _dev(ids, table)
     _i32(ids, "ids"); _i32(table, "table")
-    _need(ids.dim() == 1 and table.dim() == 2 and 0 < n_experts <= MOE_MAX_EXPERTS, f"moe_route: ids [T], table [V, top], at most {MOE_MAX_EXPERTS} experts")
-    T, top = ids.numel(), table.shape[1]
-    buf = torch.empty(2 * T * top + n_experts + 1, dtype=torch.int32, device=ids.device)
+    _need(table.dim() == 2 and 0 < n_experts <= MOE_MAX_EXPERTS, f"moe_route: table [rows, top], at most {MOE_MAX_EXPERTS} experts")
+    _need(ids is None or ids.dim() == 1, "moe_route: ids [T]")
+    T, top = (ids.numel() if ids is not None else table.shape[0]), table.shape[1]
+    buf = torch.empty(2 * T * top + n_experts + 1, dtype=torch.int32, device=table.device)
     order, where, seg = buf[:T * top], buf[T * top:2 * T * top], buf[2 * T * top:]
     _check(_lib().llogos_moe_route(_p(ids), _p(table), T, top, n_experts, _p(order), _p(seg), _p(where), _stream()), "moe_route")
     return order, seg, where
 
 
+MOE_ROUTER_FEW_ROWS = 64     # up to so many rows the router's logits are made a wave an output; beyond, by the tiled 32-bit product
+
+
+def moe_router(h: torch.Tensor, router_w: torch.Tensor, correction: Optional[torch.Tensor], n_groups: int, keep: int, top: int,
+               scale: float):
+    """A router's choice for every row of h [T, K] (any storage type): logits z = h . router_w^T in 32-bit
+    (router_w float32 [E, K]), s = softmax(z) over all E outputs, the choice's scores s + correction (float32 [E]
+    or None), of which only those in the `keep` best of n_groups equal groups of neighbouring outputs (a group's
+    score is its largest) can be chosen; the `top` largest are chosen (the lowest index among equals).
+    Returns (choice int32 [T, top], weight float32 [T, top]) with weight = s[choice] / (their sum + 1e-20) * scale."""
+    _dev(router_w, correction)
+    _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1, "moe_router: rows [T, K] on the GPU")
+    _need(router_w.dtype == torch.float32 and router_w.dim() == 2 and router_w.shape[1] == h.shape[1], "moe_router: router_w must be float32 [E, K]")
+    T, Kk = h.shape
+    E = router_w.shape[0]
+    _need(0 < top <= E <= MOE_MAX_EXPERTS, f"moe_router: top within 1..E, at most {MOE_MAX_EXPERTS} outputs")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (E,)), "moe_router: correction must be float32 [E]")
+    n_groups, keep = max(1, int(n_groups)), int(keep)
+    if n_groups > 1:
+        _need(E % n_groups == 0 and keep >= 1 and min(keep, n_groups) * (E // n_groups) >= top,
+              "moe_router: equal groups, and the kept ones must hold at least `top` outputs")
+    if T <= MOE_ROUTER_FEW_ROWS:
+        z = torch.empty((T, E), dtype=torch.float32, device=h.device)
+        _check(_lib().llogos_moe_router_logits(_p(z), _p(h), _dt(h), h.stride(0) if T > 1 else max(Kk, h.stride(0)), _p(router_w),
+                                               T, E, Kk, _stream()), "moe_router_logits")
+    else:
+        z = gemm_generic(h, router_w, None, torch.float32)
+    choice = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    weight = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    _check(_lib().llogos_moe_router_choose(_p(z), _p(correction), T, E, n_groups, keep, top, ctypes.c_float(scale), _p(choice),
+                                           _p(weight), _stream()), "moe_router_choose")
+    return choice, weight
+
+
+def moe_combine_weighted(y: torch.Tensor, where: torch.Tensor, choice: torch.Tensor, weight: torch.Tensor, n_real: int,
+                         h: torch.Tensor, shared: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [T, W]: sum_j weight[t, j] * row_j + shared[t], where row_j is the pair's row y[where[t * top + j]]
+    when choice[t, j] < n_real and the token's own row h[t] otherwise (a router output that has no matrices and
+    returns its input).  y float32 [T * top, W]; h [T, W] of any storage type; shared float32 [T, W] or parts."""
+    _dev(y, where, choice, weight)
+    _i32(where, "where"); _i32(choice, "choice")
+    _need(choice.dim() == 2 and weight.shape == choice.shape and weight.dtype == torch.float32, "moe_combine_weighted: choice and weight [T, top]")
+    T, top = choice.shape
+    _need(y.dtype == torch.float32 and y.dim() == 2 and y.shape[0] == T * top and where.numel() == T * top, "moe_combine_weighted: y float32 [T * top, W]")
+    W = y.shape[1]
+    _need(h.is_cuda and h.dim() == 2 and h.shape == (T, W) and h.stride(1) == 1, "moe_combine_weighted: h must be [T, W]")
+    parts, part_stride = 1, 0
+    if shared is not None:
+        _dev(shared)
+        parts, part_stride = _parts(shared)
+        _need(shared.dtype == torch.float32 and tuple(shared.shape[-2:]) == (T, W), "moe_combine_weighted: shared rows float32 [T, W]")
+    out = torch.empty((T, W), dtype=torch.float32, device=y.device)
+    _check(_lib().llogos_moe_combine_weighted(_p(out), _p(y), _p(where), _p(choice), _p(weight), top, int(n_real), _p(h), _dt(h),
+                                              h.stride(0) if T > 1 else max(W, h.stride(0)), _p(shared), parts,
+                                              ctypes.c_longlong(part_stride), T, W, _stream()), "moe_combine_weighted")
+    return out
+
+
 def moe_product(a: torch.Tensor, w: torch.Tensor, order: torch.Tensor, seg: torch.Tensor, top: int, gather: bool,
-                out_dtype: torch.dtype, relu2: bool = False, scale: float = 1.0) -> torch.Tensor:
+                out_dtype: torch.dtype, relu2: bool = False, scale: float = 1.0, gated: bool = False) -> torch.Tensor:
     """[P, N]: sorted row r, which belongs to the expert e whose segment holds it, is a_row(r) . w[e]^T, with
     a_row(r) = a[order[r] // top] (gather: a holds the step's token rows) or a[r] (a is sorted already);
-    w [E, N, K]; relu2 squares max(., 0) in the epilogue, scale multiplies the result."""
+    w [E, N, K]; relu2 squares max(., 0) in the epilogue, scale multiplies the result.  gated: the rows of
+    w[e] are gate and up rows in turn (gate 0, up 0, gate 1, ...) and the result is [P, N / 2], column i
+    silu(gate_i sum) * (up_i sum).  `seg` may hold more segments than w has experts: rows in those belong
+    to choices without a matrix and are left unwritten."""
     _dev(a, w, order, seg)
     _i32(order, "order"); _i32(seg, "seg")
-    _need(a.dim() == 2 and w.dim() == 3 and a.shape[1] == w.shape[2] and seg.numel() == w.shape[0] + 1, "moe_product: a [M, K], w [E, N, K]")
+    _need(a.dim() == 2 and w.dim() == 3 and a.shape[1] == w.shape[2] and seg.numel() >= w.shape[0] + 1, "moe_product: a [M, K], w [E, N, K]")
     _need(a.dtype == w.dtype, "moe_product: rows and matrices of one type")
+    _need(not (relu2 and gated), "moe_product: one epilogue at a time")
     E, N, Kk = w.shape
     P = order.numel()
     _need(gather or a.shape[0] == P, "moe_product: sorted rows must be as many as pairs")
     _need(not gather or a.shape[0] * top == P, "moe_product: token rows times choices must be the pairs")
-    out = torch.empty((P, N), dtype=out_dtype, device=a.device)
+    _need(not gated or N % 2 == 0, "moe_product: gate and up rows in turn make an even number of rows")
+    act = 2 if gated else (1 if relu2 else 0)
+    out = torch.empty((P, N // 2 if gated else N), dtype=out_dtype, device=a.device)
     if a.dtype == torch.bfloat16 and MOE_PRODUCT != "plain" and a.stride(1) == 1:
         # on the matrix cores: tiles of 16 sorted rows straight from memory for steps of few rows, tiles of 64 or
         # 128 rows through LDS where an expert's segment is long enough on average to fill them
@@ -641,12 +715,12 @@ def moe_product(a: torch.Tensor, w: torch.Tensor, order: torch.Tensor, seg: torc
         if MOE_PRODUCT in ("few", "tiles64", "tiles128"):
             form = ("few", "tiles64", "tiles128").index(MOE_PRODUCT)
         code = _lib().llogos_moe_product_bf16(_p(out), _DT[out_dtype], _p(a), _p(w), _p(order), _p(seg), E, top, 1 if gather else 0,
-                                              P, N, Kk, a.stride(0), 1 if relu2 else 0, ctypes.c_float(scale), form, _stream())
+                                              P, N, Kk, a.stride(0), act, ctypes.c_float(scale), form, _stream())
         if code != -2:
             _check(code, "moe_product")
             return out
     _check(_lib().llogos_moe_product(_p(out), _DT[out_dtype], _p(a), _dt(a), _p(w), _dt(w), _p(order), _p(seg), E, top,
-                                     1 if gather else 0, P, N, Kk, a.stride(0), 1 if relu2 else 0, ctypes.c_float(scale), _stream()),
+                                     1 if gather else 0, P, N, Kk, a.stride(0), act, ctypes.c_float(scale), _stream()),
            "moe_product")
     return out
 
@@ -688,12 +762,15 @@ def latent_prepare(ctx, kv: torch.Tensor, qfull: torch.Tensor, q_out: torch.Tens
     the rotated shared key part go to the token's key row in the cache ([rank | rot | zeros]); each
     head's rotated query part goes to q_out[t, h, rank:] ([T, heads, hd], hd the cache's row width).  With a
     value pool the latent is also stored as the token's value row."""
-    _dev(kv, qfull, q_out, norm_w, cs, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos)
+    _dev(q_out, norm_w, cs, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos)
     _i32(table, "table")
     T = ctx.n_tokens
     hd = q_out.shape[-1]
-    _need(kv.dtype == torch.float32 and kv.shape == (T, rank + rot), "latent_prepare: kv must be float32 [T, rank + rot]")
-    _need(qfull.dtype == torch.float32 and qfull.shape == (T, n_heads * (dim + rot)), "latent_prepare: q must be float32 [T, heads * (dim + rot)]")
+    # (kv and qfull may be columns of wider rows)
+    _need(kv.is_cuda and kv.dtype == torch.float32 and kv.shape == (T, rank + rot) and kv.stride(1) == 1,
+          "latent_prepare: kv must be float32 [T, rank + rot]")
+    _need(qfull.is_cuda and qfull.dtype == torch.float32 and qfull.shape == (T, n_heads * (dim + rot)) and qfull.stride(1) == 1,
+          "latent_prepare: q must be float32 [T, heads * (dim + rot)]")
     _need(q_out.shape == (T, n_heads, hd) and q_out.dtype == k_pool.dtype, "latent_prepare: q_out must be [T, heads, hd] of the cache's type")
     _need(hd % 16 == 0 and hd >= rank + rot, "latent_prepare: the cache's row is too narrow")
     _check_pools(k_pool, v_pool, 1, hd, "latent_prepare")
@@ -703,7 +780,8 @@ def latent_prepare(ctx, kv: torch.Tensor, qfull: torch.Tensor, q_out: torch.Tens
     if rot_dims:
         _need(cs is not None and cs.dtype == torch.float32 and cs.shape == (T, rot_dims // 2, 2), "latent_prepare: rotary table shape")
     _need(table.dim() == 2, "latent_prepare: page table must be [batch, pages]")
-    _check(_lib().llogos_latent_prepare(_p(kv), kv.stride(0), _p(qfull), qfull.stride(0), _p(q_out), _dt(q_out), _p(norm_w),
+    ld = lambda t_, least: t_.stride(0) if T > 1 else max(least, t_.stride(0))
+    _check(_lib().llogos_latent_prepare(_p(kv), ld(kv, rank + rot), _p(qfull), ld(qfull, n_heads * (dim + rot)), _p(q_out), _dt(q_out), _p(norm_w),
                                         ctypes.c_float(eps), _p(cs), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(ctx.tok_seq),
                                         _p(ctx.tok_pos), T, n_heads, dim, rot, rot_dims, rank, hd, _stream()), "latent_prepare")
 
@@ -755,26 +833,34 @@ def latent_attention_mfma(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: to
     return out
 
 
-def head_products(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_kn: Optional[torch.Tensor] = None) -> torch.Tensor:
+def head_products(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_kn: Optional[torch.Tensor] = None,
+                  gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t, h, :N] = w[h] . a[t, h, :K] for every head h: a [T, H, >= K] and out [T, H, >= N] may be
     views with their own row and head strides; w [H, N, K] is dense.  w_kn [H, K, N]: the same matrices
-    k-major, which steps of up to 16 rows stream instead (a kernel whose threads own an output each)."""
+    k-major, which steps of up to 16 rows stream instead (a kernel whose threads own an output each).
+    gate float32 [T, >= H] (a view of wider rows will do): head h's outputs of row t are multiplied by
+    sigmoid(gate[t, h])."""
     _need(a.is_cuda and w.is_cuda and out.is_cuda and w.is_contiguous(), "head_products: device tensors, dense w")
     _need(a.dim() == 3 and out.dim() == 3 and w.dim() == 3, "head_products: a [T, H, K], w [H, N, K], out [T, H, N]")
     T, H, K = a.shape
     N = w.shape[1]
     _need(w.shape == (H, N, K) and out.shape == (T, H, N), "head_products: shapes do not fit")
     _need(a.stride(2) == 1 and out.stride(2) == 1, "head_products: unit inner strides")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= H
+              and gate.stride(1) == 1, "head_products: gate must be float32 [T, >= H]")
+        gate_stride = gate.stride(0) if T > 1 else max(H, gate.stride(0))
     if w_kn is not None and 0 < T <= 16:
         _need(w_kn.is_cuda and w_kn.is_contiguous() and w_kn.shape == (H, K, N) and w_kn.dtype == w.dtype, "head_products: w_kn must be [H, K, N] like w")
         code = _lib().llogos_head_products_few(_p(out), _dt(out), out.stride(0), out.stride(1), _p(a), _dt(a), a.stride(0), a.stride(1),
-                                               _p(w_kn), _dt(w_kn), T, H, N, K, _stream())
+                                               _p(w_kn), _dt(w_kn), T, H, N, K, _p(gate), gate_stride, _stream())
         if code != -2:
             _check(code, "head_products_few")
             return out
     if T:
         _check(_lib().llogos_head_products(_p(out), _dt(out), out.stride(0), out.stride(1), _p(a), _dt(a), a.stride(0), a.stride(1),
-                                           _p(w), _dt(w), T, H, N, K, _stream()), "head_products")
+                                           _p(w), _dt(w), T, H, N, K, _p(gate), gate_stride, _stream()), "head_products")
     return out
 
 
@@ -1818,10 +1904,11 @@ CAPPED_PREFILL_HALVES = 0         # 0: chosen by the step; 1 or 2 sets of waves 
 
 def capped_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor, n_heads: int,
                      n_kv_heads: int, head_dim: int, v_dim: int, scale: float, softcap: float = 0.0,
-                     unit_sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     head_sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of the step's query rows q [T, n_heads * head_dim] over their sequences' pages, for keys of
-    head_dim and values of v_dim dimensions: scores bent to softcap * tanh(score / softcap) (softcap > 0), a sink of
-    score 0 in the softmax's denominator (unit_sink: float32 zeros [n_heads]), head h's output times
+    head_dim and values of v_dim dimensions: scores bent to softcap * tanh(score / softcap) (softcap > 0), a sink in
+    the softmax's denominator (head_sink float32 [n_heads]: exp(head_sink[h]) is added to head h's sums; zeros for a
+    sink of score 0), head h's output times
     sigmoid(gate[t, h]) (gate float32 [T, >= n_heads], maybe a view of wider rows).  Returns [T, n_heads * v_dim].
     bfloat16 with head sizes the matrix-core kernels take runs there; everything else in the kernel for any shape."""
     T = ctx.n_tokens
@@ -1838,14 +1925,16 @@ def capped_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
                 gate_stride = gate.stride(0) if T > 1 else max(n_heads, gate.stride(0))
             out = torch.empty((T, n_heads * v_dim), dtype=torch.bfloat16, device=q.device)
             lib = _lib()
-            sink = 1 if unit_sink is not None else 0
+            if head_sink is not None:
+                _dev(head_sink)
+                _need(head_sink.dtype == torch.float32 and head_sink.shape == (n_heads,), "attention: head_sink must be float32 [n_heads]")
             if ctx.is_decode:
                 width = table.shape[1]
                 _need(table.shape[0] == T and ctx.tok_pos.numel() == T, "attention: one table row and position a sequence")
                 ws = _attn_workspace(q.device, lib.llogos_capped_attn_decode_workspace(T, n_heads, n_kv_heads, v_dim, width))
                 code = lib.llogos_capped_attn_decode_bf16(
                     _p(out), _p(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), width, _p(ctx.tok_pos), T,
-                    n_heads, n_kv_heads, head_dim, v_dim, ctypes.c_float(scale), ctypes.c_float(softcap), sink, _p(gate),
+                    n_heads, n_kv_heads, head_dim, v_dim, ctypes.c_float(scale), ctypes.c_float(softcap), _p(head_sink), _p(gate),
                     gate_stride, _p(ws), ctypes.c_longlong(ws.numel()), _stream())
             else:
                 cu = ctx.cu_dev
@@ -1859,12 +1948,12 @@ def capped_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
                 code = lib.llogos_capped_attn_prefill_bf16(
                     _p(out), _p(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
                     ctx.batch, n_tiles, n_heads, n_kv_heads, head_dim, v_dim, ctypes.c_float(scale), ctypes.c_float(softcap),
-                    sink, _p(gate), gate_stride, int(tile_rows), int(halves), _stream())
+                    _p(head_sink), _p(gate), gate_stride, int(tile_rows), int(halves), _stream())
             if code != -2:
                 _check(code, "capped_attention")
                 return out
     return attention_generic(q, n_heads * head_dim, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos, n_heads, n_kv_heads,
-                             head_dim, scale, v_dim=v_dim, head_sink=unit_sink, softcap=softcap, gate=gate)
+                             head_dim, scale, v_dim=v_dim, head_sink=head_sink, softcap=softcap, gate=gate)
 
 
 # ----------------------------------------------------------------------------

@@ -296,3 +296,72 @@ class PostNormBlock(Block):
             h = self._close(x, d, self.ffn_norm)
             mark(ctx, "norm")
         return x, (None if self.rt.is_f32 else NormedAhead(h, None))
+
+
+@register_block("output_norm")
+class OutputNormBlock(Block):
+    """The norm stands on each sublayer's output alone, and the sublayers read the stream itself:
+
+        x <- x + mixer_norm(mixer(x));   x <- x + ffn_norm(ffn(x))
+
+    The feed-forward (with its norm) may be absent.  The stream stays float32; each closing kernel
+    (ops.kernels.sandwich_norm: the output's norm and weight, the sum with the stream) also leaves the
+    completed rows in the runtime's type for whoever reads them next, and the block hands the last such rows
+    on in place of a delta (`NormedAhead(rows, None)`: the stream is complete, and these are its own rows),
+    which a block that reads the stream itself takes up and every norm ignores.  Norms that are not RMS
+    norms over the stream's width run their own kernel, and a sum kernel adds their rows."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward comes with the norm on its output, or not at all")
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def mixers(self) -> List[Mixer]:
+        return [self.mixer]
+
+    def feed_forwards(self) -> List[FeedForward]:
+        return [self.ffn] if self.ffn is not None else []
+
+    def parts(self) -> List[Part]:
+        return [p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None]
+
+    def entry_norm(self) -> Optional[Norm]:
+        return None                      # the block's first reader takes the stream as it is
+
+    def _close(self, x: torch.Tensor, out, norm: Norm) -> torch.Tensor:
+        """x += norm(out) in place; returns the completed rows in the runtime's type."""
+        from ..ops import kernels as K
+        if isinstance(norm, RMSNorm) and x.shape[1] * 4 <= 65536:
+            if self.rt.is_f32:
+                K.sandwich_norm(x, out, norm.weight, None, norm.eps, torch.float32)
+                return x
+            return K.sandwich_norm(x, out, norm.weight, None, norm.eps, self.rt.dtype, plain_rows=True)
+        import inspect
+        a = out if (out.dim() == 2 and out.dtype == torch.float32) else K.sum_parts(out, None, torch.float32)
+        if "out_dtype" in inspect.signature(norm.forward).parameters:
+            rows = norm.forward(a, out_dtype=torch.float32)
+        else:
+            rows = norm.forward(a)
+        K.residual_add(x, rows)
+        return x if self.rt.is_f32 else K.sum_parts(x, None, self.rt.dtype)
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches):
+        from ..ops import kernels as K
+        cache = caches[0] if isinstance(caches, (list, tuple)) else caches
+        if isinstance(pending, NormedAhead) and pending.norm is None and pending.rows.dtype == self.rt.dtype:
+            h = pending.rows                                  # the block before left the stream's rows
+        else:
+            if isinstance(pending, torch.Tensor):
+                K.residual_add(x, K.sum_parts(pending, None, torch.float32))
+            h = x if self.rt.is_f32 else K.sum_parts(x, None, self.rt.dtype)
+        mark(ctx, "norm")
+        a = self.mixer.forward(ctx, h, cache)
+        mark(ctx, "mixer")
+        h = self._close(x, a, self.mixer_norm)
+        mark(ctx, "norm")
+        if self.ffn is not None:
+            d = self.ffn.forward(ctx, h)
+            mark(ctx, "feed_forward")
+            h = self._close(x, d, self.ffn_norm)
+            mark(ctx, "norm")
+        return x, (None if self.rt.is_f32 else NormedAhead(h, None))

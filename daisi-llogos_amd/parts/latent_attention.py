@@ -1,15 +1,19 @@
-"""Attention through a low-rank latent, with a learned sink in the softmax.
+"""Attention through a low-rank latent, with an optional learned sink in the softmax and an optional
+sigmoid gate on every head's output.
 
     c_q = norm(W_dq h);  q = W_uq c_q                    per head [dim unrotated | rot rotated]
+                                                         (q_rank 0: q = W_q h, no latent on the query's side)
     [c_raw | k_rot] = W_dkv h;  c = norm(c_raw)          the latent, and one rotated key part for all heads
     k_h = W_uk,h c;  v_h = W_uv,h c
     score_h(i, j) = (q_h,plain(i) . k_h(j) + q_h,rot(i) . k_rot(j)) * scale,   j <= i
-    weights = exp(score) / (sum_j exp(score) + exp(sink_h))
+    weights = exp(score) / (sum_j exp(score) [+ exp(sink_h)])
+    out = W_o [sigmoid(W_g h)_h * sum_j weights_h(i, j) v_h(j)]_h            (the gate is optional)
 
 The cache holds one row [c | k_rot] a token, which serves every head, and no values of its own.
 The scores are taken in the latent's space, q_h,plain . W_uk,h c = (W_uk,h^T q_h,plain) . c, so a
 head's query becomes [W_uk,h^T q_h,plain | q_h,rot] against the cached row, the weighted sum runs
-over latents, and W_uv,h is applied to that sum."""
+over latents, and W_uv,h is applied to that sum (the gate in that product's epilogue).  The
+projections that read h (q or dq, dkv, g) are one stacked product."""
 from __future__ import annotations
 
 from typing import Callable, List, Optional
@@ -28,13 +32,13 @@ class LatentAttention(Mixer):
 
     def __init__(self, prefix: str, hidden: int, n_heads: int, dim: int, rot_dim: int, v_dim: int, q_rank: int,
                  kv_rank: int, scale: float, eps: float, position: Optional[Rotary] = None, sink: bool = True,
-                 suffix: str = ""):
+                 suffix: str = "", head_gate: bool = False):
         self.prefix, self.hidden = prefix, int(hidden)
         self.n_heads, self.dim, self.rot_dim, self.v_dim = int(n_heads), int(dim), int(rot_dim), int(v_dim)
         self.q_rank, self.kv_rank = int(q_rank), int(kv_rank)
         self.scale, self.eps = float(scale), float(eps)
         self.position = position
-        self.has_sink = bool(sink)
+        self.has_sink, self.head_gate = bool(sink), bool(head_gate)
         if position is not None and (position.pairing != 1 or position.rot > self.rot_dim):
             raise ValueError("the rotated key part takes neighbouring pairs, at most rot_dim dimensions")
         # the cached row [latent | rotated part], widened to the pages' step of 16 dimensions
@@ -42,14 +46,22 @@ class LatentAttention(Mixer):
         if self.row > 1024:
             raise ValueError(f"a cached row of {self.row} values is more than the attention kernel takes (1024)")
         H = self.n_heads
-        self.dq = Linear([prefix + "dq"], hidden, [self.q_rank], suffix=suffix)
-        self.uq = Linear([prefix + "uq"], self.q_rank, [H * (self.dim + self.rot_dim)], suffix=suffix)
-        self.dkv = Linear([prefix + "dkv"], hidden, [self.kv_rank + self.rot_dim], suffix=suffix)
+        # what reads h beside the query's latent, stacked: [q (without a latent of its own) | dkv | g]
+        self.q_width = 0 if self.q_rank else H * (self.dim + self.rot_dim)
+        names, outs = [prefix + "dkv"], [self.kv_rank + self.rot_dim]
+        if not self.q_rank:
+            names, outs = [prefix + "q"] + names, [self.q_width] + outs
+        if self.head_gate:
+            names.append(prefix + "g")
+            outs.append(H)
+        self.inp = Linear(names, hidden, outs, suffix=suffix)
+        self.dq = Linear([prefix + "dq"], hidden, [self.q_rank], suffix=suffix) if self.q_rank else None
+        self.uq = Linear([prefix + "uq"], self.q_rank, [H * (self.dim + self.rot_dim)], suffix=suffix) if self.q_rank else None
         self.o = Linear([prefix + "o"], H * self.v_dim, [hidden], suffix=suffix)
         self.uk_t = self.uv = self.uk_kn = self.uv_kn = self.q_norm_w = self.c_norm_w = self.sink = None
 
     def _linears(self) -> List[Linear]:
-        return [self.dq, self.uq, self.dkv, self.o]
+        return [lin for lin in (self.dq, self.uq, self.inp, self.o) if lin is not None]
 
     @property
     def head_dim(self) -> int:         # (what Model.step_flops takes as the width of a head's dot products)
@@ -65,7 +77,9 @@ class LatentAttention(Mixer):
     def tensor_specs(self) -> List[TensorSpec]:
         p, H = self.prefix, self.n_heads
         specs = [s for lin in self._linears() for s in lin.tensor_specs()]
-        specs += [TensorSpec(p + "dq.norm", (self.q_rank,), "norm"), TensorSpec(p + "dkv.norm", (self.kv_rank,), "norm"),
+        if self.q_rank:
+            specs.append(TensorSpec(p + "dq.norm", (self.q_rank,), "norm"))
+        specs += [TensorSpec(p + "dkv.norm", (self.kv_rank,), "norm"),
                   TensorSpec(p + "uk", (H * self.dim, self.kv_rank), "matrix"),
                   TensorSpec(p + "uv", (H * self.v_dim, self.kv_rank), "matrix")]
         if self.has_sink:
@@ -78,7 +92,7 @@ class LatentAttention(Mixer):
             lin.bind(get, rt)
         H = self.n_heads
         f32 = lambda name: get(self.prefix + name).to(device=rt.device, dtype=torch.float32).contiguous()
-        self.q_norm_w, self.c_norm_w = f32("dq.norm"), f32("dkv.norm")
+        self.q_norm_w, self.c_norm_w = (f32("dq.norm") if self.q_rank else None), f32("dkv.norm")
         self.sink = f32("sink") if self.has_sink else None
         uk = get(self.prefix + "uk").to(device=rt.device, dtype=rt.dtype)
         # per head the transposed key matrix [rank, dim]: a query's unrotated part times it is the query in the latent's space
@@ -96,16 +110,21 @@ class LatentAttention(Mixer):
     def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
         f32, H, T = torch.float32, self.n_heads, ctx.n_tokens
         plain = lambda p: K.sum_parts(p, None, f32)          # (a product may come as partial sums of a split along k)
-        cq = plain(self.dq.product(h, f32_ok=True))
-        cq = K.rmsnorm(cq, self.q_norm_w, self.eps, self.rt.dtype)
-        q = plain(self.uq.product(cq, f32_ok=True))                               # [T, H * (dim + rot)]
-        kv = plain(self.dkv.product(h, f32_ok=True))                              # [T, rank + rot]
+        rows = plain(self.inp.product(h, f32_ok=True))                            # [T, (q) | rank + rot | (heads)]
+        kv = rows[:, self.q_width:self.q_width + self.kv_rank + self.rot_dim]
+        gate = rows[:, self.q_width + self.kv_rank + self.rot_dim:] if self.head_gate else None
+        if self.q_rank:
+            cq = plain(self.dq.product(h, f32_ok=True))
+            cq = K.rmsnorm(cq, self.q_norm_w, self.eps, self.rt.dtype)
+            q = plain(self.uq.product(cq, f32_ok=True))                           # [T, H * (dim + rot)]
+        else:
+            q = rows[:, :self.q_width]
         mark(ctx, "projections")
         cs = self.position.prepare(ctx) if self.position is not None else None
         qa = torch.empty((T, H, self.row), dtype=self.rt.dtype, device=h.device)
         K.latent_prepare(ctx, kv, q, qa, self.c_norm_w, self.eps, cs, cache.k_pool, cache.v_pool, cache.table, H, self.dim, self.rot_dim,
                          self.position.rot if self.position is not None else 0, self.kv_rank)
-        K.head_products(q.view(T, H, self.dim + self.rot_dim)[:, :, :self.dim], self.uk_t, qa[:, :, :self.kv_rank], self.uk_kn)
+        K.head_products(q.unflatten(1, (H, self.dim + self.rot_dim))[:, :, :self.dim], self.uk_t, qa[:, :, :self.kv_rank], self.uk_kn)
         mark(ctx, "rotation")
         lat = None
         if cache.v_pool is not None:
@@ -115,7 +134,7 @@ class LatentAttention(Mixer):
                                       self.scale, v_dim=self.kv_rank, head_sink=self.sink)
         mark(ctx, "attention")
         a = torch.empty((T, H, self.v_dim), dtype=self.rt.dtype, device=h.device)
-        K.head_products(lat.view(T, H, self.kv_rank), self.uv, a, self.uv_kn)
+        K.head_products(lat.view(T, H, self.kv_rank), self.uv, a, self.uv_kn, gate=gate)
         out = self.o.product(a.view(T, H * self.v_dim), f32_ok=True)
         mark(ctx, "o")
         return out

@@ -3,7 +3,7 @@
 Gate and up are one stacked product whose row is [gate | up]."""
 from __future__ import annotations
 
-from typing import Callable, List, Optional
+from typing import Callable, List, Optional, Sequence
 
 import torch
 
@@ -20,11 +20,13 @@ class SwiGLU(FeedForward):
     takes_normed_rows = True
     adds_to_residual = True
 
-    def __init__(self, prefix: str, hidden: int, intermediate: int):
+    def __init__(self, prefix: str, hidden: int, intermediate: int,
+                 names: Sequence[str] = ("gate_proj", "up_proj", "down_proj"), suffix: str = ".weight"):
+        """names, suffix: the three matrices' tensor names behind `prefix`."""
         self.prefix = prefix
         self.hidden, self.intermediate = hidden, intermediate
-        self.gate_up = Linear([prefix + "gate_proj", prefix + "up_proj"], hidden, [intermediate, intermediate], gated=True)
-        self.down = Linear([prefix + "down_proj"], intermediate, [hidden])
+        self.gate_up = Linear([prefix + names[0], prefix + names[1]], hidden, [intermediate, intermediate], gated=True, suffix=suffix)
+        self.down = Linear([prefix + names[2]], intermediate, [hidden], suffix=suffix)
 
     def tensor_specs(self) -> List[TensorSpec]:
         return self.gate_up.tensor_specs() + self.down.tensor_specs()

@@ -94,3 +94,95 @@ class TableMoE(FeedForward):
         out = K.moe_combine(y, where, self.top, shared, gate)
         mark(ctx, "combine")
         return out
+
+
+@register_feed_forward("routed_moe")
+class RoutedMoE(FeedForward):
+    """A mixture of gated experts chosen by a router, beside an optional shared expert:
+
+        z = W_router h (32-bit);  s = softmax(z) over all router outputs
+        choice scores c = s + correction; the outputs form `groups` equal groups of neighbours, a group's score is
+        its largest c, and only outputs of the `keep` best groups can be chosen; the `top` largest c are chosen
+        weights w_j = s_j / (sum of the chosen s + 1e-20) * scale
+        out = sum_j w_j expert_j(h)  +  shared(h),     expert(h) = W_down (silu(W_gate h) * (W_up h))
+
+    The last `identity` router outputs have no matrices: such an expert returns h itself.  The choice, the
+    sorting of the (token, choice) pairs by expert and the weighted sum are made on the device, so single-token
+    steps are captured and replayed.  An expert's gate and up matrices are stacked with their rows in turn
+    (gate 0, up 0, gate 1, ...), so that a gate's and an up's sum of one column meet in one thread of the
+    experts' product, which writes silu(gate) * up alone."""
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden: int, n_experts: int, top: int, intermediate: int, identity: int = 0,
+                 groups: int = 1, keep: int = 1, scale: float = 1.0, shared_intermediate: int = 0, correction: bool = True):
+        total = int(n_experts) + int(identity)
+        if not 1 <= top <= total <= K.MOE_MAX_EXPERTS:
+            raise ValueError(f"top {top} of {total} router outputs: outside 1..outputs..{K.MOE_MAX_EXPERTS}")
+        if groups < 1 or total % groups or not 1 <= keep <= groups or keep * (total // groups) < top:
+            raise ValueError(f"{groups} groups of which {keep} are kept do not fit {total} router outputs and top {top}")
+        self.prefix, self.hidden = prefix, int(hidden)
+        self.n_experts, self.identity, self.top, self.intermediate = int(n_experts), int(identity), int(top), int(intermediate)
+        self.groups, self.keep, self.scale = int(groups), int(keep), float(scale)
+        self.shared_intermediate, self.has_correction = int(shared_intermediate), bool(correction)
+        self.router_w = self.correction = self.gate_up = self.down = None
+        self.shared = None
+        if self.shared_intermediate:
+            from .mlp import SwiGLU
+            self.shared = SwiGLU(prefix + "shared.", hidden, self.shared_intermediate, names=("gate", "up", "down"), suffix="")
+
+    @property
+    def outputs(self) -> int:
+        return self.n_experts + self.identity
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        p = self.prefix
+        specs = []
+        for e in range(self.n_experts):
+            specs += [TensorSpec(f"{p}e{e}.gate", (self.intermediate, self.hidden), "matrix"),
+                      TensorSpec(f"{p}e{e}.up", (self.intermediate, self.hidden), "matrix"),
+                      TensorSpec(f"{p}e{e}.down", (self.hidden, self.intermediate), "matrix")]
+        specs.append(TensorSpec(p + "router", (self.outputs, self.hidden), "router"))
+        if self.has_correction:
+            specs.append(TensorSpec(p + "correction", (self.outputs,), "correction"))
+        if self.shared is not None:
+            specs += self.shared.tensor_specs()
+        return specs
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        p, E, F = self.prefix, self.n_experts, self.intermediate
+        if E:
+            self.gate_up = torch.empty((E, 2 * F, self.hidden), dtype=rt.dtype, device=rt.device)
+            self.down = torch.empty((E, self.hidden, F), dtype=rt.dtype, device=rt.device)
+            for e in range(E):
+                self.gate_up[e, 0::2].copy_(get(f"{p}e{e}.gate"))
+                self.gate_up[e, 1::2].copy_(get(f"{p}e{e}.up"))
+                self.down[e].copy_(get(f"{p}e{e}.down"))
+        self.router_w = get(p + "router").to(device=rt.device, dtype=torch.float32).contiguous()
+        self.correction = get(p + "correction").to(device=rt.device, dtype=torch.float32).contiguous() if self.has_correction else None
+        if self.shared is not None:
+            self.shared.bind(get, rt)
+
+    def matrix_elements(self) -> int:
+        """What a token is multiplied with: the router, its `top` experts (as if all had matrices) and the shared one."""
+        return super().matrix_elements() + self.outputs * self.hidden + 3 * self.top * self.intermediate * self.hidden
+
+    def forward(self, ctx: StepContext, h: torch.Tensor):
+        choice, weight = K.moe_router(h, self.router_w, self.correction, self.groups, self.keep, self.top, self.scale)
+        mark(ctx, "router")
+        T, W = h.shape
+        if self.n_experts:
+            order, seg, where = K.moe_route(None, choice, self.outputs)
+            act = K.moe_product(h, self.gate_up, order, seg, self.top, True, self.rt.dtype, gated=True)
+            y = K.moe_product(act, self.down, order, seg, self.top, False, torch.float32)
+        else:
+            where = torch.zeros(T * self.top, dtype=torch.int32, device=h.device)
+            y = torch.zeros((T * self.top, W), dtype=torch.float32, device=h.device)
+        mark(ctx, "experts")
+        shared = None
+        if self.shared is not None:
+            shared = _float32(self.shared.forward(ctx, h))
+            mark(ctx, "shared")
+        out = K.moe_combine_weighted(y, where, choice, weight, self.n_experts, h, shared)
+        mark(ctx, "combine")
+        return out

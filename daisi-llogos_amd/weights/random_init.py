@@ -22,9 +22,10 @@ _STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch
 
 # kinds of tensors that are drawn uniformly from a range instead of N(0, std): norm weights around
 # one, norm weights stored as offsets from one, mixing weights between 0 and 1, decay biases (the
-# decay is exp(-exp(bias + ...))), learned scores of a softmax sink, an activation's shape numbers
+# decay is exp(-exp(bias + ...))), learned scores of a softmax sink, an activation's shape numbers, a router's
+# rows (wide enough that its softmax is far from flat), the correction that joins a router's scores for the choice
 _UNIFORM = {"norm": (0.9, 1.1), "offset": (-0.1, 0.1), "unit": (0.0, 0.8), "decay": (-6.0, -0.5), "sink": (0.0, 4.0),
-            "shape": (-1.5, 0.5), "taps": (-0.5, 0.5), "bonus": (-0.5, 1.5)}
+            "shape": (-1.5, 0.5), "taps": (-0.5, 0.5), "bonus": (-0.5, 1.5), "router": (-0.06, 0.06), "correction": (-0.1, 0.1)}
 _MASK32 = 0xFFFFFFFF
 _CHUNK = {"cpu": 1 << 20, "cuda": 1 << 26}     # elements made at a time (on the CPU what stays in the caches)
 
