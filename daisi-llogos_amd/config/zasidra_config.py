@@ -154,7 +154,7 @@ def _attention(mr: ConfigReader, where: str, before: list) -> ZasidraAttention:
         if own.kv_from is not None:
             raise ConfigError(f"{where}.mixer: kv_from names layer {m.kv_from}, which has no keys and values of its own")
         if (own.kv_heads, own.dim, own.vdim, own.rot) != (m.kv_heads, m.dim, m.vdim, m.rot):
-            raise ConfigError(f"{where}.mixer: a layer that reads layer {m.kv_from}'s keys and values must have its kv_heads, dim, vdim and rot")
+            raise ConfigError(f"{where}.mixer: kv_from names layer {m.kv_from}, whose kv_heads, dim, vdim or rot differ from this layer's")
     return m
 
 

@@ -11,8 +11,8 @@ from .wkv import WKV
 from .latent_attention import LatentAttention
 from .mlp import ActivatedMLP, SwiGLU
 from .capped_attention import CappedAttention
-from .moe import TableMoE
+from .moe import RoutedMoE, TableMoE
 from .loop import LoopEntry
 from .rglru import RGLRU
 from .diff_attention import DiffAttention
-from .block import ParallelBlock, PostNormBlock, PreNormBlock, SandwichBlock
+from .block import OutputNormBlock, ParallelBlock, PostNormBlock, PreNormBlock, SandwichBlock

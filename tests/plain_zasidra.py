@@ -213,7 +213,7 @@ def part(tensors: dict, prefix: str) -> dict:
 def forward(cfg: dict, tensors: dict, tokens, streams: list = None) -> np.ndarray:
     """Logits [T, vocab] of one whole sequence.  streams: a list that receives the stream after every layer."""
     eps = cfg["norm"]["eps"]
-    x = tensors["embed"][np.asarray(tokens)] * cfg["embedding"]["scale"]
+    x = tensors["embed"][np.asarray(tokens)] * (cfg.get("embedding") or {}).get("scale", 1.0)
     positions = np.arange(len(tokens))
     kept = {}
     for i, L in enumerate(cfg["layers"]):
@@ -236,3 +236,13 @@ def forward(cfg: dict, tensors: dict, tokens, streams: list = None) -> np.ndarra
         if streams is not None:
             streams.append(x.copy())
     return offset_norm(x, tensors["final.norm"], eps) @ tensors["head"].T
+
+
+def generate_greedy(cfg: dict, tensors: dict, prompt, n: int) -> list:
+    """n tokens, each the first largest logit after everything before it (the whole sequence is run again each time)."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        tok = int(np.argmax(forward(cfg, tensors, seq)[-1]))
+        out.append(tok)
+        seq.append(tok)
+    return out
