@@ -195,15 +195,44 @@ def batodra_config(width, layers, vocab, ff):
             "layers": [(rec, win, rec, dif)[i % 4] for i in range(layers)], "torch_dtype": "bfloat16"}
 
 
+def zasidra_config(width, layers, vocab, ff):
+    """Layers of real sizes: latent attention and grouped-query attention in turn, every second attention layer reading
+    the keys and values of the one before it; heads of 128 dimensions (keys and values), four query heads a key/value
+    head, half of a head rotated with stretched frequencies; latents of 512; the first layer's feed-forward dense, the
+    others' a mixture with 16 router outputs in 4 groups of which 2 are kept, 14 experts with matrices and 2 that return
+    their input, 2 a token, each expert a quarter and the shared one half as wide as the dense decoder's feed-forward
+    (the dense decoder's matrix bytes a token)."""
+    heads = width // 128
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 2},
+           "router": {"experts": 14, "identity": 2, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 2}}}
+    att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+           "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    lat = {"type": "latent_attention", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "kv_rank": 512, "scale": 128 ** -0.5}}
+    out = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff} if i == 0 else moe
+        if i % 2 == 0:
+            out.append(dict(lat, mlp=mlp))
+        else:
+            out.append({"type": "attention", "mixer": dict(att, kv_from=i - 2) if i % 4 == 3 else att, "mlp": mlp})
+    return {"architecture": "Zasidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "layers": out, "torch_dtype": "bfloat16"}
+
+
 def moe_bytes_read(model, ids) -> int:
     """Bytes of weights that a step with the token ids `ids` reads: as step_weight_bytes, but of a layer's experts
-    only those that the layer's table names for these ids."""
+    only those that the layer's table names for these ids, or that its router chose in the last step that was
+    run part by part (a router's choice depends on the stream, not on the ids alone)."""
     total = model.step_weight_bytes()
     for e in model.schedule:
         for f in model.layers[e.layer].feed_forwards():
-            if hasattr(f, "n_experts"):
+            if hasattr(f, "table"):
                 experts = (f.up.numel() + f.down.numel()) * f.up.element_size()
                 chosen = len(set(f.table[list(ids)].reshape(-1).tolist()))
+                total -= experts - experts * chosen // f.n_experts
+            elif getattr(f, "probed", None) and f.n_experts:
+                experts = (f.gate_up.numel() + f.down.numel()) * f.down.element_size()
+                chosen = len({c for c in f.probed["choice"].reshape(-1).tolist() if c < f.n_experts})
                 total -= experts - experts * chosen // f.n_experts
     return total
 
@@ -256,6 +285,9 @@ def compare_designs(args) -> int:
             eng.step([(x, toks(args.prompt_len)) for x in slots], want="last")
             ids = toks(batch)                                     # a token of its own for every sequence (an expert choice of its own)
             step = lambda: eng.step([(x, [t]) for x, t in zip(slots, ids)], want="last", borrow=True)
+            if args.design == "zasidra" and label.startswith("zasidra"):
+                # a step run part by part leaves every router's choice behind: the experts that such a step reads
+                eng.step([(x, [t]) for x, t in zip(slots, ids)], want="last", probe=llogos.StepProbe())
             for _ in range(args.warmup):
                 step()
             dt = timed(lambda: [step() for _ in range(args.steps)], repeat=2) / args.steps
@@ -281,6 +313,8 @@ def compare_designs(args) -> int:
                      num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), tie_word_embeddings=True)
         if args.design == "zogurax":
             other = zogurax_config(width, layers, vocab, ff)
+        elif args.design == "zasidra":
+            other = zasidra_config(width, layers, vocab, ff)
         elif args.design == "batodra":
             other = batodra_config(width, layers, vocab, ff * 3 // 2)
         else:
@@ -290,6 +324,9 @@ def compare_designs(args) -> int:
         if args.design == "batodra":
             # the other design that mixes recurrent layers with attention, at the same sizes
             entry["nipulorn"] = measure(f"nipulorn {name}", nipulorn_config(width, layers, vocab, ff * 3 // 2), vocab)
+        if args.design == "zasidra":
+            # the other design with attention behind a norm over the whole projection and a mixture of experts
+            entry["zogurax"] = measure(f"zogurax {name}", zogurax_config(width, layers, vocab, ff), vocab)
         entry["dense"] = measure(f"dense {name}", dense, vocab)
         record["sizes"].append(entry)
     print(json.dumps(record), flush=True)
@@ -298,7 +335,7 @@ def compare_designs(args) -> int:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["nipulorn", "zogurax", "batodra"], default=None,
+    ap.add_argument("--design", choices=["nipulorn", "zogurax", "batodra", "zasidra"], default=None,
                     help="instead of the default run: this design beside the dense decoder at equal sizes (prefill, decode, parts)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=248)   # + 8 warm-up = 256 new tokens

@@ -15,13 +15,14 @@
 // qfull [T, ldq] float holds per head [dim | rot]; the head's rot part is rotated the same way
 // and written to q_out[t, h, rank .. rank + rot), zeros behind it up to hd.
 // With a value pool (the matrix cores' attention reads values in their own operand order) the
-// latent is stored there too, as dimensions 0..rank-1 of the token's value row.
+// latent is stored there too, as dimensions 0..rank-1 of the token's value row.  With c_out the normed latents are
+// also left as plain rows [T, rank] (for a caller that multiplies them with the heads' key and value matrices).
 template <typename T>
 __global__ void latent_prepare_kernel(const float* __restrict__ kv, int ldkv, const float* __restrict__ qfull, int ldq,
                                       T* __restrict__ q_out, const float* __restrict__ norm_w, float eps,
                                       const float2* __restrict__ cs, T* __restrict__ k_pool, T* __restrict__ v_pool, PagedKV cache,
                                       const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-                                      int n_heads, int dim, int rot, int rot_dims, int rank, int hd) {
+                                      int n_heads, int dim, int rot, int rot_dims, int rank, int hd, T* __restrict__ c_out) {
     __shared__ float red[16];
     const int t = blockIdx.x, tid = threadIdx.x;
     const int seq = tok_seq[t], pos = tok_pos[t];
@@ -39,6 +40,7 @@ __global__ void latent_prepare_kernel(const float* __restrict__ kv, int ldkv, co
         const float v = row[i] * inv * norm_w[i];
         store_f32(page + page_key_offset(in_page, i, hd), v);
         if (v_pool) store_f32(v_pool + page_at + page_value_offset(in_page, i), v);     // the latent again, as a value
+        if (c_out) store_f32(c_out + (size_t)t * rank + i, v);
     }
     for (int i = tid; i < hd - rank; i += blockDim.x) {
         float v = 0.f;
@@ -72,17 +74,17 @@ __global__ void latent_prepare_kernel(const float* __restrict__ kv, int ldkv, co
 LLOGOS_EXPORT int llogos_latent_prepare(const float* kv, int ldkv, const float* qfull, int ldq, void* q_out, int dtype,
                                         const float* norm_w, float eps, const void* cs, void* k_pool, void* v_pool,
                                         const int* table, int table_stride, const int* tok_seq, const int* tok_pos,
-                                        int T, int n_heads, int dim, int rot, int rot_dims, int rank, int hd,
+                                        int T, int n_heads, int dim, int rot, int rot_dims, int rank, int hd, void* c_out,
                                         hipStream_t stream) {
     if (T <= 0 || n_heads <= 0 || dim < 0 || rot < 0 || rank <= 0 || hd < rank + rot || hd % 16) return LLOGOS_BAD_ARGUMENT;
     if (rot_dims < 0 || rot_dims > rot || rot_dims % 2 || ldkv < rank + rot || ldq < n_heads * (dim + rot)) return LLOGOS_BAD_ARGUMENT;
     PagedKV cache{table, table_stride, 1, hd};
     if (dtype == DT_F32)
         latent_prepare_kernel<float><<<T, 256, 0, stream>>>(kv, ldkv, qfull, ldq, (float*)q_out, norm_w, eps, (const float2*)cs,
-                                                            (float*)k_pool, (float*)v_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
+                                                            (float*)k_pool, (float*)v_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd, (float*)c_out);
     else if (dtype == DT_BF16)
         latent_prepare_kernel<bf16_t><<<T, 256, 0, stream>>>(kv, ldkv, qfull, ldq, (bf16_t*)q_out, norm_w, eps, (const float2*)cs,
-                                                             (bf16_t*)k_pool, (bf16_t*)v_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
+                                                             (bf16_t*)k_pool, (bf16_t*)v_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd, (bf16_t*)c_out);
     else
         return LLOGOS_BAD_ARGUMENT;
     return LLOGOS_LAUNCH_CHECK();

@@ -215,29 +215,85 @@ LLOGOS_EXPORT int llogos_moe_combine(float* out, const float* y, const int* wher
 }
 
 // ---------------------------------------------------------------- a router
-// z[t, e] = w[e, :] . a[t, :] in 32-bit for steps of few rows: a wave a (token, output), lanes along k, the lanes'
-// sums added by the wave's reduction.  w float32 [E, K]; a [T, lda] of any storage type.
-template <typename TA>
+// z[t, e] = w[e, :] . a[t, :] in 32-bit.  A wave takes R token rows and G router outputs: its lanes go along k four
+// values at a time (lane l takes k = 4 l .. 4 l + 3, then 256 further on), every value of a row serves the G outputs
+// and every value of w the R rows; the lanes' sums are added by the wave's reduction at the end.  The order of an
+// output's additions depends on k alone, so a row's logits are the same bits in a step of one row and of thousands.
+// w float32 [E, K]; a [T, lda] of any storage type.  VEC: K, lda and the pointers allow 16-byte (8-byte) loads.
+template <typename TA> struct RouterRow4;
+template <> struct RouterRow4<float> {
+    static __device__ __forceinline__ float4 load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+};
+template <> struct RouterRow4<bf16_t> {
+    static __device__ __forceinline__ float4 load(const bf16_t* p) {
+        const uint2 u = *reinterpret_cast<const uint2*>(p);
+        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                           __uint_as_float(u.y & 0xffff0000u));
+    }
+};
+
+template <typename TA, int R, int G, bool VEC>
 __global__ __launch_bounds__(256) void moe_router_logits_kernel(float* __restrict__ z, const TA* __restrict__ a, int lda,
-                                                                const float* __restrict__ w, int E, int K) {
+                                                                const float* __restrict__ w, int T, int E, int K) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const int e = blockIdx.x * 4 + wave, t = blockIdx.y;
-    if (e >= E) return;
-    const TA* ar = a + (size_t)t * lda;
-    const float* wr = w + (size_t)e * K;
-    float acc = 0.f;
-    for (int k = lane; k < K; k += kWave) acc = fmaf(load_f32(ar + k), wr[k], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) z[(size_t)t * E + e] = acc;
+    const int t0 = (blockIdx.x * 4 + wave) * R, e0 = blockIdx.y * G;
+    if (t0 >= T) return;
+    float acc[R][G];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int g = 0; g < G; ++g) acc[r][g] = 0.f;
+    for (int k = 4 * lane; k < K; k += 4 * kWave) {
+        float4 av[R], wv[G];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const TA* p = a + (size_t)min(t0 + r, T - 1) * lda + k;
+            if (VEC) av[r] = RouterRow4<TA>::load(p);
+            else av[r] = make_float4(load_f32(p), k + 1 < K ? load_f32(p + 1) : 0.f, k + 2 < K ? load_f32(p + 2) : 0.f,
+                                     k + 3 < K ? load_f32(p + 3) : 0.f);
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float* p = w + (size_t)min(e0 + g, E - 1) * K + k;
+            if (VEC) wv[g] = *reinterpret_cast<const float4*>(p);
+            else wv[g] = make_float4(p[0], k + 1 < K ? p[1] : 0.f, k + 2 < K ? p[2] : 0.f, k + 3 < K ? p[3] : 0.f);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float s = acc[r][g];
+                s = fmaf(av[r].x, wv[g].x, s);
+                s = fmaf(av[r].y, wv[g].y, s);
+                s = fmaf(av[r].z, wv[g].z, s);
+                s = fmaf(av[r].w, wv[g].w, s);
+                acc[r][g] = s;
+            }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float s = wave_sum(acc[r][g]);
+            if (lane == 0 && t0 + r < T && e0 + g < E) z[(size_t)(t0 + r) * E + e0 + g] = s;
+        }
 }
 
 LLOGOS_EXPORT int llogos_moe_router_logits(float* z, const void* a, int a_dtype, int lda, const float* w, int T, int E, int K,
                                            hipStream_t stream) {
-    if (T <= 0 || E <= 0 || K <= 0 || lda < K) return LLOGOS_BAD_ARGUMENT;
-    dim3 grid((E + 3) / 4, T);
-    if (a_dtype == DT_F32) moe_router_logits_kernel<float><<<grid, 256, 0, stream>>>(z, (const float*)a, lda, w, E, K);
-    else if (a_dtype == DT_BF16) moe_router_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>(z, (const bf16_t*)a, lda, w, E, K);
-    else return LLOGOS_BAD_ARGUMENT;
+    if (T <= 0 || E <= 0 || K <= 0 || lda < K || (a_dtype != DT_F32 && a_dtype != DT_BF16)) return LLOGOS_BAD_ARGUMENT;
+    const int elt = a_dtype == DT_F32 ? 4 : 2;
+    const bool vec = K % 4 == 0 && lda % 4 == 0 && (uintptr_t)a % (4 * elt) == 0 && (uintptr_t)w % 16 == 0;
+    // few rows: a row a wave and four outputs, so that the step has waves enough; many: four rows a wave and eight outputs
+    const bool few = T <= 64;
+    const int R = few ? 1 : 4, G = few ? 4 : 8;
+    dim3 grid((T + 4 * R - 1) / (4 * R), (E + G - 1) / G);
+#define RL(TA, R_, G_, V) moe_router_logits_kernel<TA, R_, G_, V><<<grid, 256, 0, stream>>>(z, (const TA*)a, lda, w, T, E, K)
+#define RLV(TA, R_, G_) do { if (vec) RL(TA, R_, G_, true); else RL(TA, R_, G_, false); } while (0)
+    if (a_dtype == DT_F32) { if (few) RLV(float, 1, 4); else RLV(float, 4, 8); }
+    else { if (few) RLV(bf16_t, 1, 4); else RLV(bf16_t, 4, 8); }
+#undef RLV
+#undef RL
     return LLOGOS_LAUNCH_CHECK();
 }
 

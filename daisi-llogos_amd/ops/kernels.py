@@ -347,21 +347,27 @@ def qkv_prepare(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype:
                 head_dim: int, v_dim: int, q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
                 temp_coef: float, temp_every: int, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
                 table: Optional[torch.Tensor], writes: bool = True, cs: Optional[torch.Tensor] = None, rot: int = 0,
-                pairing: int = 0) -> torch.Tensor:
+                pairing: int = 0, kv_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """From projected rows [q | k | v | ...] (float32 [T, >= W] or partial sums [parts, T, >= W], plus `bias`
     [W], W = n_heads * head_dim + n_kv_heads * (head_dim + v_dim)): an RMS norm over the whole of q and of
     k where a weight is given ([n_heads * head_dim], [n_kv_heads * head_dim]), then the rotation of the first
     `rot` dimensions of every head of q and k by the table `cs` [T, rot / 2, 2] (pairing 0: dimension i with
     i + rot / 2, 1: 2i with 2i + 1), the query's factor 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1);
     q comes back [T, n_heads * head_dim] in `out_dtype`, k and v go to their pages.  writes False: only q is
-    made (the rows then need hold no more than q)."""
+    made (the rows then need hold no more than q).  kv_rows: float32 [T, >= n_kv_heads * (head_dim + v_dim)] rows
+    [k | v] in one part, for keys and values that were not projected together with q (qkv then holds q alone)."""
     _need(qkv.is_cuda and qkv.dtype == torch.float32 and qkv.stride(-1) == 1, "qkv_prepare: float32 rows on the GPU")
     _dev(bias, q_norm_w, k_norm_w, table, ctx.tok_seq, ctx.tok_pos)
     parts, part_stride = _parts(qkv)
     T = qkv.shape[-2]
     Wq, Wk, Wv = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_dim
-    width = Wq + ((Wk + Wv) if writes else 0)
+    width = Wq + ((Wk + Wv) if (writes and kv_rows is None) else 0)
     _need(qkv.shape[-1] >= width and T == ctx.n_tokens, f"qkv_prepare: rows of at least {width} values, one a token")
+    kv_stride = 0
+    if kv_rows is not None:
+        _need(writes and kv_rows.is_cuda and kv_rows.dtype == torch.float32 and kv_rows.dim() == 2 and kv_rows.shape[0] == T
+              and kv_rows.shape[1] >= Wk + Wv and kv_rows.stride(1) == 1, f"qkv_prepare: kv_rows must be float32 [T, >= {Wk + Wv}]")
+        kv_stride = kv_rows.stride(0) if T > 1 else max(Wk + Wv, kv_rows.stride(0))
     _need(rot % 2 == 0 and 0 <= rot <= head_dim and pairing in (0, 1), "qkv_prepare: the rotated width must be even and within a head")
     if rot:
         _dev(cs)
@@ -387,7 +393,7 @@ def qkv_prepare(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype:
         n_kv_heads if writes else 0, head_dim, v_dim, kd, vd, _p(q_norm_w), _p(k_norm_w), ctypes.c_float(eps),
         ctypes.c_float(temp_coef), int(temp_every), _p(cs) if rot else None, int(rot), int(pairing), _p(k_pool) if writes else None, _p(v_pool) if writes else None,
         _p(table) if writes else None, table.stride(0) if (writes and table is not None) else 0, _p(ctx.tok_seq), _p(ctx.tok_pos),
-        T, _stream()), "qkv_prepare")
+        _p(kv_rows), kv_stride, T, _stream()), "qkv_prepare")
     return q_out
 
 
@@ -630,9 +636,6 @@ def moe_route(ids: Optional[torch.Tensor], table: torch.Tensor, n_experts: int):
     return order, seg, where
 
 
-MOE_ROUTER_FEW_ROWS = 64     # up to so many rows the router's logits are made a wave an output; beyond, by the tiled 32-bit product
-
-
 def moe_router(h: torch.Tensor, router_w: torch.Tensor, correction: Optional[torch.Tensor], n_groups: int, keep: int, top: int,
                scale: float):
     """A router's choice for every row of h [T, K] (any storage type): logits z = h . router_w^T in 32-bit
@@ -651,12 +654,9 @@ def moe_router(h: torch.Tensor, router_w: torch.Tensor, correction: Optional[tor
     if n_groups > 1:
         _need(E % n_groups == 0 and keep >= 1 and min(keep, n_groups) * (E // n_groups) >= top,
               "moe_router: equal groups, and the kept ones must hold at least `top` outputs")
-    if T <= MOE_ROUTER_FEW_ROWS:
-        z = torch.empty((T, E), dtype=torch.float32, device=h.device)
-        _check(_lib().llogos_moe_router_logits(_p(z), _p(h), _dt(h), h.stride(0) if T > 1 else max(Kk, h.stride(0)), _p(router_w),
-                                               T, E, Kk, _stream()), "moe_router_logits")
-    else:
-        z = gemm_generic(h, router_w, None, torch.float32)
+    z = torch.empty((T, E), dtype=torch.float32, device=h.device)
+    _check(_lib().llogos_moe_router_logits(_p(z), _p(h), _dt(h), h.stride(0) if T > 1 else max(Kk, h.stride(0)), _p(router_w),
+                                           T, E, Kk, _stream()), "moe_router_logits")
     choice = torch.empty((T, top), dtype=torch.int32, device=h.device)
     weight = torch.empty((T, top), dtype=torch.float32, device=h.device)
     _check(_lib().llogos_moe_router_choose(_p(z), _p(correction), T, E, n_groups, keep, top, ctypes.c_float(scale), _p(choice),
@@ -757,11 +757,12 @@ def moe_combine(y: torch.Tensor, where: torch.Tensor, top: int, shared: Optional
 # ----------------------------------------------------------------------------
 def latent_prepare(ctx, kv: torch.Tensor, qfull: torch.Tensor, q_out: torch.Tensor, norm_w: torch.Tensor, eps: float,
                    cs: Optional[torch.Tensor], k_pool: torch.Tensor, v_pool: Optional[torch.Tensor], table: torch.Tensor,
-                   n_heads: int, dim: int, rot: int, rot_dims: int, rank: int) -> None:
+                   n_heads: int, dim: int, rot: int, rot_dims: int, rank: int, c_out: Optional[torch.Tensor] = None) -> None:
     """From kv float32 [T, rank + rot] and qfull float32 [T, heads * (dim + rot)]: the normed latent and
     the rotated shared key part go to the token's key row in the cache ([rank | rot | zeros]); each
     head's rotated query part goes to q_out[t, h, rank:] ([T, heads, hd], hd the cache's row width).  With a
-    value pool the latent is also stored as the token's value row."""
+    value pool the latent is also stored as the token's value row, and with c_out ([T, rank] of the cache's type)
+    as plain rows."""
     _dev(q_out, norm_w, cs, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos)
     _i32(table, "table")
     T = ctx.n_tokens
@@ -780,10 +781,13 @@ def latent_prepare(ctx, kv: torch.Tensor, qfull: torch.Tensor, q_out: torch.Tens
     if rot_dims:
         _need(cs is not None and cs.dtype == torch.float32 and cs.shape == (T, rot_dims // 2, 2), "latent_prepare: rotary table shape")
     _need(table.dim() == 2, "latent_prepare: page table must be [batch, pages]")
+    if c_out is not None:
+        _dev(c_out)
+        _need(c_out.shape == (T, rank) and c_out.dtype == k_pool.dtype, "latent_prepare: c_out must be [T, rank] of the cache's type")
     ld = lambda t_, least: t_.stride(0) if T > 1 else max(least, t_.stride(0))
     _check(_lib().llogos_latent_prepare(_p(kv), ld(kv, rank + rot), _p(qfull), ld(qfull, n_heads * (dim + rot)), _p(q_out), _dt(q_out), _p(norm_w),
                                         ctypes.c_float(eps), _p(cs), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(ctx.tok_seq),
-                                        _p(ctx.tok_pos), T, n_heads, dim, rot, rot_dims, rank, hd, _stream()), "latent_prepare")
+                                        _p(ctx.tok_pos), T, n_heads, dim, rot, rot_dims, rank, hd, _p(c_out), _stream()), "latent_prepare")
 
 
 LATENT_MFMA_MAX_ROW = 576

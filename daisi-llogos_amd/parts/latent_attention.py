@@ -13,7 +13,13 @@ The cache holds one row [c | k_rot] a token, which serves every head, and no val
 The scores are taken in the latent's space, q_h,plain . W_uk,h c = (W_uk,h^T q_h,plain) . c, so a
 head's query becomes [W_uk,h^T q_h,plain | q_h,rot] against the cached row, the weighted sum runs
 over latents, and W_uv,h is applied to that sum (the gate in that product's epilogue).  The
-projections that read h (q or dq, dkv, g) are one stacked product."""
+projections that read h (q or dq, dkv, g) are one stacked product.
+
+Whole prompts in bfloat16 whose head shapes the matrix cores' attention takes, and that have no rotated
+part, go the other way round: the step's latents are multiplied with all heads' key and value matrices at
+once (one product of the library's kind), the keys and values go to pages of the step's own, and the
+prompt kernel of the attention with keys and values a head runs on them: a quarter or less of the
+arithmetic of scores and sums over latents, on the faster kernel.  The cache still gets the latents alone."""
 from __future__ import annotations
 
 from typing import Callable, List, Optional
@@ -59,6 +65,8 @@ class LatentAttention(Mixer):
         self.uq = Linear([prefix + "uq"], self.q_rank, [H * (self.dim + self.rot_dim)], suffix=suffix) if self.q_rank else None
         self.o = Linear([prefix + "o"], H * self.v_dim, [hidden], suffix=suffix)
         self.uk_t = self.uv = self.uk_kn = self.uv_kn = self.q_norm_w = self.c_norm_w = self.sink = None
+        self.ukv = None              # [uk ; uv] stacked by rows, for whole prompts
+        self.prompt_rows = 128       # steps of at least so many tokens that are all whole prompts make keys and values a head
 
     def _linears(self) -> List[Linear]:
         return [lin for lin in (self.dq, self.uq, self.inp, self.o) if lin is not None]
@@ -101,11 +109,51 @@ class LatentAttention(Mixer):
         # the same two sets of matrices k-major, for steps of few rows (a few MB a layer)
         self.uk_kn = uk.view(H, self.dim, self.kv_rank).contiguous()
         self.uv_kn = self.uv.transpose(1, 2).contiguous()
+        if self._heads_on_matrix_cores():
+            self.ukv = torch.cat([uk, self.uv.view(H * self.v_dim, self.kv_rank)], dim=0).contiguous()
         if self.position is not None and getattr(self.position, "inv_freq", None) is None:
             self.position.bind(get, rt)
 
     def matrix_elements(self) -> int:
         return super().matrix_elements() + self.n_heads * self.kv_rank * (self.dim + self.v_dim)
+
+    def _heads_on_matrix_cores(self) -> bool:
+        """Whether whole prompts can run as attention with keys and values a head (see the module's text)."""
+        return self.rt.dtype == torch.bfloat16 and self.rot_dim == 0 and not self.q_rank and self.dim in (64, 96, 128) \
+            and self.v_dim in (64, 80, 96, 128)
+
+    @staticmethod
+    def _prompt_pages(ctx: StepContext):
+        """Pages of the step's own for whole prompts: (number of pages, table int32 [batch, pages of the longest]), sequence
+        after sequence; made once a step on the device from the step's token offsets."""
+        made = ctx.shared.get("prompt_pages")
+        if made is None:
+            lens = [ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch)]
+            pages = [-(-n // K.PAGE_TOKENS) for n in lens]
+            counts = (ctx.cu_dev[1:] - ctx.cu_dev[:-1] + (K.PAGE_TOKENS - 1)) // K.PAGE_TOKENS
+            first = torch.cumsum(counts, 0) - counts
+            table = (first[:, None] + torch.arange(max(pages), device=first.device)[None, :]).to(torch.int32).contiguous()
+            made = ctx.shared["prompt_pages"] = (sum(pages), table)
+        return made
+
+    def _forward_prompt(self, ctx: StepContext, rows: torch.Tensor, kv: torch.Tensor, gate, cache: LayerCache) -> torch.Tensor:
+        f32, H, T = torch.float32, self.n_heads, ctx.n_tokens
+        qa = torch.empty((T, H, self.row), dtype=self.rt.dtype, device=rows.device)       # (no rotated part: nothing is written)
+        c = torch.empty((T, self.kv_rank), dtype=self.rt.dtype, device=rows.device)
+        K.latent_prepare(ctx, kv, rows[:, :self.q_width], qa, self.c_norm_w, self.eps, None, cache.k_pool, cache.v_pool, cache.table,
+                         H, self.dim, 0, 0, self.kv_rank, c_out=c)
+        keys_values = K.sum_parts(K.gemm_product(c, self.ukv, self.rt.dtype, f32_ok=True), None, f32)     # [T, H * (dim + v_dim)]
+        mark(ctx, "rotation")
+        n_pages, table = self._prompt_pages(ctx)
+        k_pool = torch.empty((n_pages, H, K.PAGE_TOKENS * self.dim), dtype=self.rt.dtype, device=rows.device)
+        v_pool = torch.empty((n_pages, H, K.PAGE_TOKENS * self.v_dim), dtype=self.rt.dtype, device=rows.device)
+        q = K.qkv_prepare(ctx, rows, None, self.rt.dtype, H, H, self.dim, self.v_dim, None, None, self.eps, 0.0, 1, k_pool, v_pool,
+                          table, kv_rows=keys_values)
+        a = K.capped_attention(ctx, q, k_pool, v_pool, table, H, H, self.dim, self.v_dim, self.scale, 0.0, self.sink, gate)
+        mark(ctx, "attention")
+        out = self.o.product(a, f32_ok=True)
+        mark(ctx, "o")
+        return out
 
     def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
         f32, H, T = torch.float32, self.n_heads, ctx.n_tokens
@@ -120,6 +168,9 @@ class LatentAttention(Mixer):
         else:
             q = rows[:, :self.q_width]
         mark(ctx, "projections")
+        if self.ukv is not None and not ctx.is_decode and not ctx.in_graph and T >= self.prompt_rows and ctx.cu_dev is not None \
+                and not any(ctx.starts):
+            return self._forward_prompt(ctx, rows, kv, gate, cache)
         cs = self.position.prepare(ctx) if self.position is not None else None
         qa = torch.empty((T, H, self.row), dtype=self.rt.dtype, device=h.device)
         K.latent_prepare(ctx, kv, q, qa, self.c_norm_w, self.eps, cs, cache.k_pool, cache.v_pool, cache.table, H, self.dim, self.rot_dim,

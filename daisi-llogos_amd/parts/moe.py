@@ -9,6 +9,7 @@ experts' matrices are stacked ([experts, ff, width] and [experts, width, ff]); t
 pairs are sorted by expert and each expert's rows multiplied tile by tile."""
 from __future__ import annotations
 
+import os
 from typing import Callable, List, Optional
 
 import torch
@@ -110,8 +111,19 @@ class RoutedMoE(FeedForward):
     sorting of the (token, choice) pairs by expert and the weighted sum are made on the device, so single-token
     steps are captured and replayed.  An expert's gate and up matrices are stacked with their rows in turn
     (gate 0, up 0, gate 1, ...), so that a gate's and an up's sum of one column meet in one thread of the
-    experts' product, which writes silu(gate) * up alone."""
+    experts' product, which writes silu(gate) * up alone.
+
+    The shared expert depends on h alone, so in steps of few rows, whose kernels are short and wait for one another,
+    it is queued on a second stream beside the router and the chosen experts (inside a captured step the two become
+    branches of the graph); both streams meet before the weighted sum.  Every use of the second stream begins by
+    waiting for the first, so memory that either stream's allocator hands out again is no longer read by the other.
+    It pays where the shared expert's matrices are large (8 layers at batch 8 and 1: 4,096 wide with 176 MB of them
+    2,429 -> 2,335 us and 1,529 -> 1,470 us a step; 2,048 wide with 50 MB 1,457 -> 1,469 and 1,012 -> 1,037), so it is
+    taken from `side_bytes` of shared matrices on.  `LLOGOS_PARALLEL_STREAMS=0` keeps everything on one stream."""
     graph_safe = True
+    side_rows = 0 if os.environ.get("LLOGOS_PARALLEL_STREAMS", "1") == "0" else 64     # steps of up to so many rows use the second stream
+    side_bytes = 64 << 20        # ... when the shared expert's matrices take at least so many bytes
+    _side_streams = {}
 
     def __init__(self, prefix: str, hidden: int, n_experts: int, top: int, intermediate: int, identity: int = 0,
                  groups: int = 1, keep: int = 1, scale: float = 1.0, shared_intermediate: int = 0, correction: bool = True):
@@ -126,6 +138,7 @@ class RoutedMoE(FeedForward):
         self.shared_intermediate, self.has_correction = int(shared_intermediate), bool(correction)
         self.router_w = self.correction = self.gate_up = self.down = None
         self.shared = None
+        self.probed = None          # {"choice": int32 [T, top]} of the last step that was run part by part (measurements)
         if self.shared_intermediate:
             from .mlp import SwiGLU
             self.shared = SwiGLU(prefix + "shared.", hidden, self.shared_intermediate, names=("gate", "up", "down"), suffix="")
@@ -168,8 +181,20 @@ class RoutedMoE(FeedForward):
         return super().matrix_elements() + self.outputs * self.hidden + 3 * self.top * self.intermediate * self.hidden
 
     def forward(self, ctx: StepContext, h: torch.Tensor):
+        shared, side = None, None
+        if self.shared is not None and h.shape[0] <= self.side_rows and (ctx is None or ctx.probe is None) and h.is_cuda \
+                and 3 * self.shared_intermediate * self.hidden * h.element_size() >= self.side_bytes:
+            main = torch.cuda.current_stream(h.device)
+            side = self._side_streams.get(h.device)
+            if side is None:
+                side = self._side_streams[h.device] = torch.cuda.Stream(device=h.device)
+            side.wait_stream(main)                       # h is there
+            with torch.cuda.stream(side):
+                shared = _float32(self.shared.forward(ctx, h))
         choice, weight = K.moe_router(h, self.router_w, self.correction, self.groups, self.keep, self.top, self.scale)
         mark(ctx, "router")
+        if ctx is not None and ctx.probe is not None:
+            self.probed = {"choice": choice}
         T, W = h.shape
         if self.n_experts:
             order, seg, where = K.moe_route(None, choice, self.outputs)
@@ -179,8 +204,9 @@ class RoutedMoE(FeedForward):
             where = torch.zeros(T * self.top, dtype=torch.int32, device=h.device)
             y = torch.zeros((T * self.top, W), dtype=torch.float32, device=h.device)
         mark(ctx, "experts")
-        shared = None
-        if self.shared is not None:
+        if side is not None:
+            torch.cuda.current_stream(h.device).wait_stream(side)
+        elif self.shared is not None:
             shared = _float32(self.shared.forward(ctx, h))
             mark(ctx, "shared")
         out = K.moe_combine_weighted(y, where, choice, weight, self.n_experts, h, shared)

@@ -259,9 +259,14 @@ LATENTS = [(3, 24, 40, 48, 56), (5, 16, 8, 20, 40), (2, 40, 24, 24, 72), (4, 64,
            (1, 8, 8, 8, 16)]
 
 
+PIECES = [(60, 9, 1), (1, 1, 1), (1, 1, 1), (3, 58, 0), (1, 1, 0), (2, 0, 0), (64, 0, 0), (1, 0, 0), (17, 0, 0)]
+WHOLE = [(148, 68, 3), (1, 1, 0), (1, 1, 0)]          # prompts whole in one step (keys and values a head where the shapes allow), then single tokens
+
+
 @pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("cuts", [PIECES, WHOLE])
 @pytest.mark.parametrize("shape", LATENTS)
-def test_the_gated_latent_attention_alone_in_pieces(dtype, shape):
+def test_the_gated_latent_attention_alone_in_pieces(dtype, shape, cuts, monkeypatch):
     heads, dk, dv, rank, hidden = shape
     rng = np.random.default_rng(heads * 10 + rank)
     # scores that spread over some units whatever the sizes: sharp, and still within what bfloat16 queries resolve
@@ -284,7 +289,11 @@ def test_the_gated_latent_attention_alone_in_pieces(dtype, shape):
         v_pool[4] = float("nan")
     pages = {0: [7, 2, 5], 1: [0, 8], 2: [3]}
     got = [np.zeros((n, hidden)) for n in lengths]
-    cuts = [(60, 9, 1), (1, 1, 1), (1, 1, 1), (3, 58, 0), (1, 1, 0), (2, 0, 0), (64, 0, 0), (1, 0, 0), (17, 0, 0)]
+    by_head = cuts is WHOLE and dtype == "bfloat16" and dk in (64, 96, 128) and dv in (64, 80, 96, 128)
+    ran = []
+    if by_head:                                                # the whole prompts must take the way over keys and values a head
+        keep = mix._forward_prompt
+        monkeypatch.setattr(mix, "_forward_prompt", lambda *a, **k: (ran.append(1), keep(*a, **k))[1])
     for seqs, lo, hi in _steps(lengths, cuts):
         ctx = _ctx(mix.rt, hi, [b - a for a, b in zip(lo, hi)], [0, 1, 2][:len(seqs)])
         table = np.full((len(seqs), 3), -1, dtype=np.int32)
@@ -300,6 +309,7 @@ def test_the_gated_latent_attention_alone_in_pieces(dtype, shape):
     for i, (g, w_) in enumerate(zip(got, want)):
         assert np.isfinite(g).all()
         assert np.abs(g - w_).max() <= (2 if dtype == "bfloat16" else 1) * PART_TOL[dtype] * max(1.0, np.abs(w_).max()), f"sequence {i}"
+    assert len(ran) == (1 if by_head else 0)
     no_gate = pz.latent_attention(h[0], dict(pz.part(plain, "m."), g=np.zeros((heads, hidden))), m, 1e-5)
     assert np.abs(no_gate - want[0]).max() > 100 * PART_TOL["float32"] * np.abs(want[0]).max()      # the gate is no trifle here
 
@@ -434,8 +444,8 @@ def test_the_first_tokens_one_by_one_and_portions_down_to_two_tokens(name, dtype
 @pytest.mark.parametrize("name", ["zas_a", "zas_c"])
 def test_unequal_batches_against_each_alone_with_slots_and_pages_used_again(name, dtype):
     eng = H.engine(name, dtype, max_tokens=448, n_slots=3)              # 7 pages: the second batch needs the first one's
-    for round_, lens in enumerate([(130, 9, 70), (200, 3, 66)]):
-        seqs = [H.tokens(name, n + 6, 10 * round_ + i) for i, n in enumerate(lens)]
+    for turn, lens in enumerate([(130, 9, 70), (200, 3, 66)]):
+        seqs = [H.tokens(name, n + 6, 10 * turn + i) for i, n in enumerate(lens)]
         slots = [eng.alloc_slot() for _ in seqs]
         assert slots == [0, 1, 2]
         got = [[] for _ in seqs]
@@ -456,7 +466,7 @@ def test_unequal_batches_against_each_alone_with_slots_and_pages_used_again(name
             eng.free_slot(slots[i])
         for i, t in enumerate(seqs):
             g = np.concatenate(got[i])
-            H.close(g, H.plain_logits(name, t, dtype=dtype)[:len(g)], dtype, f"{name} round {round_} sequence {i}")
+            H.close(g, H.plain_logits(name, t, dtype=dtype)[:len(g)], dtype, f"{name} batch {turn} sequence {i}")
     assert eng.cache.free_pages() == [7] * len(eng.cache.groups)
 
 
@@ -474,6 +484,30 @@ def test_long_decoding_replayed_and_launched(name, dtype):
         outs[graphs] = np.concatenate(got)
         H.close(outs[graphs], want, dtype, f"long decoding, graphs {graphs}")
     assert np.array_equal(outs[True], outs[False])              # a replayed step is the launched step
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_the_shared_expert_on_a_second_stream_changes_no_bit(dtype, monkeypatch):
+    """Steps of few rows queue the shared expert beside the router and the chosen experts; with everything on one
+    stream the same kernels run one after the other.  Unequal batches, prompts of few rows and single tokens, replayed
+    and launched."""
+    name = "zas_a"
+    seqs = [H.tokens(name, 40, 30 + i) for i in range(3)]
+    outs = {}
+    monkeypatch.setattr(P.RoutedMoE, "side_bytes", 0)          # (a toy model's shared expert is too small to be worth a stream)
+    for rows in (64, 0):
+        monkeypatch.setattr(P.RoutedMoE, "side_rows", rows)
+        for graphs in (True, False):
+            eng = H.engine(name, dtype, use_graphs=graphs)
+            slots = [eng.alloc_slot() for _ in seqs]
+            got = [_np(eng.step([(s, list(t[:n])) for s, t, n in zip(slots, seqs, (20, 3, 9))], want="all"))]
+            for step in range(12):
+                got.append(_np(eng.step([(s, [t[n + step]]) for s, t, n in zip(slots, seqs, (20, 3, 9))], want="all")))
+            outs[(rows, graphs)] = np.concatenate(got)
+    first = outs[(64, True)]
+    assert all(np.array_equal(first, o) for o in outs.values())
+    want = np.concatenate([H.plain_logits(name, t, dtype=dtype)[:n] for t, n in zip(seqs, (20, 3, 9))])
+    H.close(first[:32], want, dtype, "two streams")
 
 
 def test_far_keys_the_sinks_another_layers_keys_and_the_outputs_without_matrices_decide_and_are_there():
