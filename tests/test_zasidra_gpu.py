@@ -109,12 +109,25 @@ def test_the_closing_kernel_norms_the_output_adds_it_and_leaves_the_rows(width, 
     assert np.abs(_np(xt) - want).max() <= 2e-5 * np.abs(want).max()
 
 
+def _closing(kind, y, w, eps):
+    if kind == "rms":
+        return pz.offset_norm(y, w, eps)
+    y = np.asarray(y, dtype=np.float64)                        # a layer norm with a weight and no bias
+    d = y - y.mean(axis=-1, keepdims=True)
+    return d / np.sqrt((d * d).mean(axis=-1, keepdims=True) + eps) * w
+
+
+@pytest.mark.parametrize("kind", ["rms", "layer"])
 @pytest.mark.parametrize("dtype", H.DTYPES)
-def test_a_block_of_the_design_with_toy_parts(dtype):
-    """x + N1(mixer(x)), then + N2(ff(x)), with a layer's real norms around a dense feed-forward on both places."""
+def test_a_block_of_the_design_with_toy_parts(dtype, kind):
+    """x + N1(mixer(x)), then + N2(ff(x)), with a dense feed-forward; the closing norms are the design's own (one kernel
+    closes a sublayer) or norms of another kind (their own kernel, then a sum)."""
     rng = np.random.default_rng(3)
     W, T = 40, 7
-    norm = lambda n: P.RMSNorm(name=n, width=W, eps=1e-5, offset=1.0, suffix="")
+    if kind == "rms":
+        norm = lambda n: P.RMSNorm(name=n, width=W, eps=1e-5, offset=1.0, suffix="")
+    else:
+        norm = lambda n: P.LayerNorm(name=n, width=W, eps=1e-5, suffix="")
     ff = P.SwiGLU(prefix="f.", hidden=W, intermediate=24, names=("gate", "up", "down"), suffix="")
 
     class Doubler(P.Mixer):                                    # a mixer without tensors: twice its input
@@ -126,8 +139,8 @@ def test_a_block_of_the_design_with_toy_parts(dtype):
     xt = torch.tensor(x, dtype=torch.float32, device=DEV)
     out, pending = blk.forward(None, xt, None, [P.LayerCache()])
     h = _rounded(x, dtype)
-    want = x + pz.offset_norm(2.0 * h, plain["n1"], 1e-5)
-    want = want + pz.offset_norm(pz.gated_ff(_rounded(want, dtype), plain["f.gate"], plain["f.up"], plain["f.down"]), plain["n2"], 1e-5)
+    want = x + _closing(kind, 2.0 * h, plain["n1"], 1e-5)
+    want = want + _closing(kind, pz.gated_ff(_rounded(want, dtype), plain["f.gate"], plain["f.up"], plain["f.down"]), plain["n2"], 1e-5)
     assert np.abs(_np(out) - want).max() <= PART_TOL[dtype] * np.abs(want).max()
     if dtype == "float32":
         assert pending is None
@@ -294,6 +307,14 @@ def test_the_gated_latent_attention_alone_in_pieces(dtype, shape, cuts, monkeypa
     if by_head:                                                # the whole prompts must take the way over keys and values a head
         keep = mix._forward_prompt
         monkeypatch.setattr(mix, "_forward_prompt", lambda *a, **k: (ran.append(1), keep(*a, **k))[1])
+        fresh = torch.empty
+
+        def poisoned(*a, **k):                                 # the step's own pages start as NaN: what is not written is not read
+            t = fresh(*a, **k)
+            if t.dtype == torch.bfloat16 and t.dim() == 3:
+                t.fill_(float("nan"))
+            return t
+        monkeypatch.setattr(torch, "empty", poisoned)
     for seqs, lo, hi in _steps(lengths, cuts):
         ctx = _ctx(mix.rt, hi, [b - a for a, b in zip(lo, hi)], [0, 1, 2][:len(seqs)])
         table = np.full((len(seqs), 3), -1, dtype=np.int32)
